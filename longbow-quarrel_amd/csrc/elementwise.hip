@@ -343,6 +343,10 @@ extern "C" int lq_cast(const void* in, int in_dtype, void* out, int out_dtype, l
     cast_kernel<float, bf16_t><<<blocks, threads, 0, stream>>>((const float*)in, (bf16_t*)out, n);
   else if (in_dtype == LQ_BF16 && out_dtype == LQ_F32)
     cast_kernel<bf16_t, float><<<blocks, threads, 0, stream>>>((const bf16_t*)in, (float*)out, n);
+  else if (in_dtype == LQ_F32 && out_dtype == LQ_F32)  // (a copy)
+    cast_kernel<float, float><<<blocks, threads, 0, stream>>>((const float*)in, (float*)out, n);
+  else if (in_dtype == LQ_BF16 && out_dtype == LQ_BF16)
+    cast_kernel<bf16_t, bf16_t><<<blocks, threads, 0, stream>>>((const bf16_t*)in, (bf16_t*)out, n);
   else
     LQ_REQUIRE(false, "cast: unsupported pair %d -> %d", in_dtype, out_dtype);
   LQ_CHECK_LAUNCH("cast");
@@ -953,6 +957,52 @@ __global__ __launch_bounds__(256) void rmsnorm_residual_kernel(float* __restrict
     if (rounded != nullptr) rounded[base + i] = from_f32<T>(v);
   }
 }
+// The norm on a sublayer's result and the norm ahead of the next sublayer in one pass over a row:
+//   y = sum_i scale_i piece_i;   x += y / sqrt(mean(y^2) + eps) * w;   (x += extra;)
+//   (h = x / sqrt(mean(x^2) + next_eps) * next_w, in the next reader's dtype.)
+// The pieces' sum is taken in the order of the pieces; both sums of squares are the block's fixed tree.
+struct NormPieces {
+  const float* y[4];
+  float scale[4];
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void postnorm_residual_kernel(float* __restrict__ x, NormPieces in, int n_in,
+                                                                const float* __restrict__ w, float eps,
+                                                                const float* __restrict__ extra,
+                                                                const float* __restrict__ next_w, float next_eps,
+                                                                T* __restrict__ h, int width) {
+  __shared__ float red[16];
+  const long long base = (long long)blockIdx.x * width;
+  auto summed = [&](int i) -> float {
+    float v = in.scale[0] * in.y[0][base + i];
+#pragma unroll
+    for (int p = 1; p < 4; ++p)
+      if (p < n_in) v = fmaf(in.scale[p], in.y[p][base + i], v);
+    return v;
+  };
+  float acc = 0.f;
+  for (int i = threadIdx.x; i < width; i += 256) {
+    const float v = summed(i);
+    acc = fmaf(v, v, acc);
+  }
+  const float inv = 1.f / sqrtf(block_sum(acc, red) / (float)width + eps);
+  float acc2 = 0.f;
+  for (int i = threadIdx.x; i < width; i += 256) {
+    float v = x[base + i] + summed(i) * inv * w[i];
+    if (extra != nullptr) v += extra[base + i];
+    x[base + i] = v;
+    acc2 = fmaf(v, v, acc2);
+  }
+  if (h == nullptr) return;
+  const float inv2 = 1.f / sqrtf(block_sum(acc2, red) / (float)width + next_eps);
+  for (int i = threadIdx.x; i < width; i += 256) h[base + i] = from_f32<T>(x[base + i] * inv2 * next_w[i]);
+}
+
+__global__ __launch_bounds__(256) void scale_kernel(float* __restrict__ x, float s, long long n) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) x[i] *= s;
+}
 }  // namespace
 
 extern "C" int lq_bigram_add(float* x, const void* table, int table_dtype, const int* tokens, int* last, long long buckets,
@@ -981,5 +1031,34 @@ extern "C" int lq_rmsnorm_residual(float* x, const float* y, const float* w, flo
     rmsnorm_residual_kernel<bf16_t><<<rows, 256, 0, stream>>>(x, y, w, eps, (bf16_t*)rounded, width);
   else LQ_REQUIRE(false, "rmsnorm_residual: unknown dtype %d", rounded_dtype);
   LQ_CHECK_LAUNCH("rmsnorm_residual");
+  return 0;
+}
+
+// y: `pieces` dense float32 [rows, width] tensors `piece_stride` entries apart, each with its scale (at most 4);
+// extra (or null) [rows, width] is added to x after the normed result; next_w (or null) with h (or null): the next
+// norm's weight and where its result goes.
+extern "C" int lq_postnorm_residual(float* x, const float* y, int pieces, long long piece_stride, float s0, float s1,
+                                    float s2, float s3, const float* w, float eps, const float* extra,
+                                    const float* next_w, float next_eps, void* h, int h_dtype, int rows, int width,
+                                    hipStream_t stream) {
+  LQ_REQUIRE(rows > 0 && width > 0, "postnorm_residual: rows %d and width %d must be positive", rows, width);
+  LQ_REQUIRE(pieces >= 1 && pieces <= 4, "postnorm_residual: %d pieces (1 to 4)", pieces);
+  LQ_REQUIRE(x && y && w && ((h == nullptr) == (next_w == nullptr)), "postnorm_residual: null pointer");
+  NormPieces in;
+  const float sc[4] = {s0, s1, s2, s3};
+  for (int i = 0; i < 4; ++i) in.y[i] = y + (i < pieces ? i : 0) * piece_stride, in.scale[i] = sc[i];
+  if (h == nullptr || h_dtype == LQ_F32)
+    postnorm_residual_kernel<float><<<rows, 256, 0, stream>>>(x, in, pieces, w, eps, extra, next_w, next_eps, (float*)h, width);
+  else if (h_dtype == LQ_BF16)
+    postnorm_residual_kernel<bf16_t><<<rows, 256, 0, stream>>>(x, in, pieces, w, eps, extra, next_w, next_eps, (bf16_t*)h, width);
+  else LQ_REQUIRE(false, "postnorm_residual: unknown dtype %d", h_dtype);
+  LQ_CHECK_LAUNCH("postnorm_residual");
+  return 0;
+}
+
+extern "C" int lq_scale(float* x, float s, long long n, hipStream_t stream) {
+  LQ_REQUIRE(x && n > 0, "scale: bad arguments");
+  scale_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(x, s, n);
+  LQ_CHECK_LAUNCH("scale");
   return 0;
 }

@@ -62,6 +62,61 @@ __global__ __launch_bounds__(128) void rotary_kernel(const float* __restrict__ s
   }
 }
 
+// Queries, keys and values of a step's rows, from the 32-bit result of their one product to what the attention
+// kernel and the cache read.  src [rows, (H + G) D + G V]: H query heads, G key heads, G value heads.  Of every query
+// and key head the first `dims` entries are rotated as in `rotary_kernel`; then, with norm_eps >= 0, the whole head
+// is divided by its root mean square over D (eps inside the root); values pass.  One workgroup a row; a wavefront
+// takes a head at a time (its sum of squares is the wavefront's fixed tree, so it depends on the row alone).
+template <typename T>
+__global__ __launch_bounds__(256) void rotary_qkv_kernel(const float* __restrict__ src, int lds_, T* __restrict__ q_out,
+                                                         int ldq, T* __restrict__ k_out, int ldk, T* __restrict__ v_out,
+                                                         int ldv, int H, int G, int D, int V, int dims, int interleaved,
+                                                         const double* __restrict__ freqs, float mag, float norm_eps,
+                                                         const int* __restrict__ row_pos) {
+  extern __shared__ float cs[];  // cos[dims / 2], sin[dims / 2]
+  const int r = blockIdx.x, half = dims / 2;
+  const int p = row_pos[r];
+  for (int j = threadIdx.x; j < half; j += blockDim.x) {
+    const double a = (double)p * freqs[j];
+    const double n = rint(a * 0.15915494309189533577);
+    double rem = fma(-n, 6.283185307179586232, a);
+    rem = fma(-n, 2.4492935982947064e-16, rem);
+    float sn, c;
+    sincosf((float)rem, &sn, &c);
+    cs[j] = c * mag;
+    cs[half + j] = sn * mag;
+  }
+  __syncthreads();
+  const float* s = src + (long long)r * lds_;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, waves = blockDim.x >> 6;
+  for (int h = wave; h < H + G; h += waves) {
+    const float* v = s + h * D;
+    T* o = h < H ? q_out + (long long)r * ldq + h * D : k_out + (long long)r * ldk + (h - H) * D;
+    auto turned = [&](int i) -> float {
+      if (i >= dims) return v[i];
+      int j, mate;
+      bool first;
+      if (interleaved) j = i >> 1, first = !(i & 1), mate = i ^ 1;
+      else first = i < half, j = first ? i : i - half, mate = first ? i + half : i - half;
+      const float c = cs[j], sn = cs[half + j];
+      return first ? v[i] * c - v[mate] * sn : v[i] * c + v[mate] * sn;
+    };
+    float inv = 1.f;
+    if (norm_eps >= 0.f) {
+      float ss = 0.f;
+      for (int i = lane; i < D; i += 64) {
+        const float t = turned(i);
+        ss = fmaf(t, t, ss);
+      }
+      inv = 1.f / sqrtf(wave_sum(ss) / (float)D + norm_eps);
+    }
+    for (int i = lane; i < D; i += 64) o[i] = from_f32<T>(turned(i) * inv);
+  }
+  const float* vs = s + (H + G) * D;
+  T* vo = v_out + (long long)r * ldv;
+  for (int e = threadIdx.x; e < G * V; e += blockDim.x) vo[e] = from_f32<T>(vs[e]);
+}
+
 // A product a head: out[r, h ohs + n] = sum_k x[r, h K + k] w[h, n, k], bfloat16 operands on
 // v_mfma_f32_16x16x16_bf16 (exact products, 32-bit sums).  A workgroup of four wavefronts takes 64 rows by 64
 // columns of one head; a wavefront 16 rows by the 64 columns, its operands straight from memory (a head's weight
@@ -134,6 +189,32 @@ extern "C" int lq_rotary(const float* src, int lds_, void* out, int out_dtype, i
                                                             interleaved, freqs, magnitude, row_pos);
   else LQ_REQUIRE(false, "rotary: unknown dtype %d", out_dtype);
   LQ_CHECK_LAUNCH("rotary");
+  return 0;
+}
+
+// src [rows, (heads + kv_heads) * key_dim + kv_heads * value_dim] float32 (stride lds_): queries, keys, values.
+// dims = 0: no rotation (freqs may be null); norm_eps < 0: no norm.
+extern "C" int lq_rotary_qkv(const float* src, int lds_, void* q_out, int ldq, void* k_out, int ldk, void* v_out, int ldv,
+                             int out_dtype, int rows, int heads, int kv_heads, int key_dim, int value_dim, int dims,
+                             int interleaved, const double* freqs, float magnitude, float norm_eps, const int* row_pos,
+                             hipStream_t stream) {
+  LQ_REQUIRE(rows > 0 && heads > 0 && kv_heads > 0 && key_dim > 0 && value_dim > 0, "rotary_qkv: rows %d, heads %d and %d, sizes %d and %d",
+             rows, heads, kv_heads, key_dim, value_dim);
+  LQ_REQUIRE(dims >= 0 && dims % 2 == 0 && dims <= key_dim && dims <= 8192, "rotary_qkv: %d rotated entries of %d", dims, key_dim);
+  LQ_REQUIRE(lds_ >= (heads + kv_heads) * key_dim + kv_heads * value_dim && ldq >= heads * key_dim && ldk >= kv_heads * key_dim &&
+                 ldv >= kv_heads * value_dim, "rotary_qkv: a row stride is smaller than its row");
+  LQ_REQUIRE(src && q_out && k_out && v_out && row_pos && (dims == 0 || freqs), "rotary_qkv: null pointer");
+  const size_t lds_bytes = (size_t)dims * sizeof(float);
+  if (out_dtype == LQ_F32)
+    rotary_qkv_kernel<float><<<rows, 256, lds_bytes, stream>>>(src, lds_, (float*)q_out, ldq, (float*)k_out, ldk, (float*)v_out,
+                                                               ldv, heads, kv_heads, key_dim, value_dim, dims, interleaved,
+                                                               freqs, magnitude, norm_eps, row_pos);
+  else if (out_dtype == LQ_BF16)
+    rotary_qkv_kernel<bf16_t><<<rows, 256, lds_bytes, stream>>>(src, lds_, (bf16_t*)q_out, ldq, (bf16_t*)k_out, ldk,
+                                                                (bf16_t*)v_out, ldv, heads, kv_heads, key_dim, value_dim, dims,
+                                                                interleaved, freqs, magnitude, norm_eps, row_pos);
+  else LQ_REQUIRE(false, "rotary_qkv: unknown dtype %d", out_dtype);
+  LQ_CHECK_LAUNCH("rotary_qkv");
   return 0;
 }
 

@@ -6,24 +6,55 @@ namespace {
 
 // One thread a row: s = sigmoid(z), the `top` largest win (the lower index on a tie); route[r, e] = the expert's
 // weight (its score, or its share of the chosen scores), -1 for an expert that was not chosen.
+// With `correction` the experts are chosen by s + correction[e]; the weights stay the scores s.  With `groups` > 1
+// the experts form that many equal groups of neighbours; a group's mark is the sum of its two largest choice scores
+// (of its one, in groups of one), and only experts of the `keep` groups with the largest marks (the lower index on a
+// tie) can be chosen.
 __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__ z, int ldz, float* __restrict__ route,
-                                                       int rows, int E, int top, int renorm) {
+                                                       int rows, int E, int top, int renorm,
+                                                       const float* __restrict__ correction, int groups, int keep) {
   const int r = blockIdx.x * 64 + threadIdx.x;
   if (r >= rows) return;
   const float* zr = z + (long long)r * ldz;
   float* out = route + (long long)r * E;
   for (int e = 0; e < E; ++e) out[e] = -1.f;
+  auto score = [&](int e) { return 1.f / (1.f + expf(-zr[e])); };
+  auto choice = [&](int e) { return correction != nullptr ? score(e) + correction[e] : score(e); };
+  unsigned long long kept = ~0ull;  // bit g: group g may be chosen from
+  const int per = groups > 1 ? E / groups : E;
+  if (groups > 1 && keep < groups) {
+    kept = 0ull;
+    for (int n = 0; n < keep; ++n) {
+      int best = -1;
+      float bm = 0.f;
+      for (int g = 0; g < groups; ++g) {
+        if ((kept >> g) & 1ull) continue;
+        float a = -INFINITY, b = -INFINITY;  // the group's two largest choice scores
+        for (int e = g * per; e < (g + 1) * per; ++e) {
+          const float v = choice(e);
+          if (v > a) b = a, a = v;
+          else if (v > b) b = v;
+        }
+        const float mark = per > 1 ? a + b : a;
+        if (best < 0 || mark > bm) best = g, bm = mark;
+      }
+      if (best < 0) break;
+      kept |= 1ull << best;
+    }
+  }
   float total = 0.f;
   for (int k = 0; k < top; ++k) {
     int best = -1;
     float bz = 0.f;
     for (int e = 0; e < E; ++e) {
       if (out[e] >= 0.f) continue;  // chosen already
-      const float v = 1.f / (1.f + expf(-zr[e]));  // scores are compared, not logits: equal scores are a tie
+      if (groups > 1 && !((kept >> (e / per)) & 1ull)) continue;
+      const float v = choice(e);  // scores are compared, not logits: equal scores are a tie
       if (best < 0 || v > bz) best = e, bz = v;
     }
     if (best < 0) break;
-    out[best] = bz == bz ? bz : 0.f;
+    const float w = score(best);
+    out[best] = w == w ? w : 0.f;
     total += out[best];
   }
   if (renorm && total > 0.f)
@@ -33,11 +64,13 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__
 
 // gu [rows, E, 2, ff] (gate then up of every expert), route [rows, E]; out [rows, E, ff]:
 // g = min(w gate, limit), u = clamp(w up, -limit, limit), y = g sigmoid(1.702 g) (u + 1) for a chosen expert (its
-// weight w on what it read: `on_input`; otherwise w multiplies y), 0 for the others.
+// weight w on what it read: `on_input`; otherwise w multiplies y), 0 for the others.  `plain_silu`: the expert is
+// y = silu(gate) up without clamps.
 template <typename T>
 __global__ __launch_bounds__(256) void moe_glu_kernel(const float* __restrict__ gu, long long ldg,
                                                       const float* __restrict__ route, T* __restrict__ out,
-                                                      long long ldo, int E, int ff, float limit, int on_input) {
+                                                      long long ldo, int E, int ff, float limit, int on_input,
+                                                      int plain_silu) {
   const int r = blockIdx.y;
   const int i = blockIdx.x * 256 + threadIdx.x;
   if (i >= E * ff) return;
@@ -47,9 +80,14 @@ __global__ __launch_bounds__(256) void moe_glu_kernel(const float* __restrict__ 
   if (w >= 0.f) {
     const float* p = gu + r * ldg + (long long)e * 2 * ff;
     const float s = on_input ? w : 1.f;
-    const float g = fminf(p[c] * s, limit);
-    const float u = fminf(fmaxf(p[ff + c] * s, -limit), limit);
-    y = g / (1.f + expf(-1.702f * g)) * (u + 1.f);
+    if (plain_silu) {
+      const float g = p[c] * s;
+      y = g / (1.f + expf(-g)) * (p[ff + c] * s);
+    } else {
+      const float g = fminf(p[c] * s, limit);
+      const float u = fminf(fmaxf(p[ff + c] * s, -limit), limit);
+      y = g / (1.f + expf(-1.702f * g)) * (u + 1.f);
+    }
     if (!on_input) y *= w;
   }
   out[r * ldo + i] = from_f32<T>(y);
@@ -128,17 +166,20 @@ __global__ __launch_bounds__(256) void moe_scatter_kernel(const float* __restric
 }  // namespace
 
 extern "C" int lq_moe_route(const float* z, int ldz, float* route, int rows, int experts, int top, int renormalize,
-                            hipStream_t stream) {
+                            const float* correction, int groups, int keep, hipStream_t stream) {
+  LQ_REQUIRE(groups >= 0 && (groups <= 1 || (groups <= 64 && experts % groups == 0 && keep >= 1 && keep <= groups)),
+             "moe_route: %d experts in %d groups of which %d are kept", experts, groups, keep);
   LQ_REQUIRE(rows > 0 && experts > 0 && top >= 1 && top <= experts && ldz >= experts, "moe_route: rows %d, %d of %d experts",
              rows, top, experts);
   LQ_REQUIRE(z && route, "moe_route: null pointer");
-  moe_route_kernel<<<lq_ceil_div(rows, 64), 64, 0, stream>>>(z, ldz, route, rows, experts, top, renormalize);
+  moe_route_kernel<<<lq_ceil_div(rows, 64), 64, 0, stream>>>(z, ldz, route, rows, experts, top, renormalize, correction,
+                                                             groups, keep);
   LQ_CHECK_LAUNCH("moe_route");
   return 0;
 }
 
 extern "C" int lq_moe_glu(const float* gu, long long ldg, const float* route, void* out, int out_dtype, long long ldo,
-                          int rows, int experts, int ff, float limit, int on_input, hipStream_t stream) {
+                          int rows, int experts, int ff, float limit, int on_input, int plain_silu, hipStream_t stream) {
   LQ_REQUIRE(rows > 0 && experts > 0 && ff > 0 && (long long)experts * ff <= 0x7fffffff, "moe_glu: rows %d, experts %d, inner %d",
              rows, experts, ff);
   LQ_REQUIRE(ldg >= 2ll * experts * ff && ldo >= (long long)experts * ff, "moe_glu: a row stride is smaller than its row");
@@ -148,10 +189,10 @@ extern "C" int lq_moe_glu(const float* gu, long long ldg, const float* route, vo
     dim3 grid(lq_ceil_div(experts * ff, 256), nr);
     if (out_dtype == LQ_F32)
       moe_glu_kernel<float><<<grid, 256, 0, stream>>>(gu + r0 * ldg, ldg, route + (long long)r0 * experts,
-                                                      (float*)out + r0 * ldo, ldo, experts, ff, limit, on_input);
+                                                      (float*)out + r0 * ldo, ldo, experts, ff, limit, on_input, plain_silu);
     else if (out_dtype == LQ_BF16)
       moe_glu_kernel<bf16_t><<<grid, 256, 0, stream>>>(gu + r0 * ldg, ldg, route + (long long)r0 * experts,
-                                                       (bf16_t*)out + r0 * ldo, ldo, experts, ff, limit, on_input);
+                                                       (bf16_t*)out + r0 * ldo, ldo, experts, ff, limit, on_input, plain_silu);
     else LQ_REQUIRE(false, "moe_glu: unknown dtype %d", out_dtype);
   }
   LQ_CHECK_LAUNCH("moe_glu");

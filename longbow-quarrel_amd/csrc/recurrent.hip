@@ -66,14 +66,20 @@ __global__ __launch_bounds__(256) void add_scaled_kernel(float* __restrict__ x, 
   x[i] += scale * d;
 }
 
-// out[r, c] = act(gu[r, c]) * gu[r, I + c]
+// out[r, c] = act(gu[r, c] + bias[c]) * (gu[r, I + c] + bias[I + c]); behind the I results `tail` more columns, a
+// one and then zeros: with the next product's bias as one more column of its weight, that product adds the bias itself
 template <typename TI, typename TO>
 __global__ __launch_bounds__(256) void glu_kernel(const TI* __restrict__ gu, int ld, TO* __restrict__ out, int ldo,
-                                                  int I, int act) {
+                                                  int I, int act, const float* __restrict__ bias, int tail) {
   const int r = blockIdx.y;
   const int c = blockIdx.x * 256 + threadIdx.x;
-  if (c >= I) return;
-  const float g = to_f32(gu[(long long)r * ld + c]), u = to_f32(gu[(long long)r * ld + I + c]);
+  if (c >= I + tail) return;
+  if (c >= I) {
+    store_as<TO>(out + (long long)r * ldo + c, c == I ? 1.f : 0.f);
+    return;
+  }
+  float g = to_f32(gu[(long long)r * ld + c]), u = to_f32(gu[(long long)r * ld + I + c]);
+  if (bias != nullptr) g += bias[c], u += bias[I + c];
   store_as<TO>(out + (long long)r * ldo + c, activate(g, act) * u);
 }
 
@@ -717,25 +723,176 @@ __global__ __launch_bounds__(256) void gla_chain_kernel(float* __restrict__ stat
   state[((long long)seq_slot[b] * heads + h) * PN + idx] = cur;
 }
 
+// Gated delta rule with a decay for every key channel: S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;
+// o = S^T q, with q and k unit vectors (made so by `unit_heads_kernel`), beta = sigmoid(raw) and
+// g = exp(-exp(A_log_h) softplus(z + bias)) for every key channel of every head, made of its logit where the chunk is
+// staged.  (ScanShape: groups = q/k heads, N = key size, P = value size; the state [slots, heads, P, N].)  The
+// staging is that of the gated linear attention scan (q, k and the decays of a chunk of tokens in LDS, two buffers
+// taking turns), with one more number a token, beta.
+constexpr int dch_tokens(int np, int th, int ln) {
+  const int by_regs = 24 * th / (3 * np), by_lds = 8192 / (3 * np + 2 * (th / ln) + 1);
+  const int t = by_regs < by_lds ? by_regs : by_lds;
+  return t >= 16 ? 16 : t >= 8 ? 8 : t >= 4 ? 4 : t >= 2 ? 2 : 1;
+}
+
+template <int LN, int SLAB, int TH>
+__global__ __launch_bounds__(TH) void delta_channel_scan_kernel(const float* __restrict__ q, int ldq,
+                                                                 const float* __restrict__ k, int ldk,
+                                                                 const float* __restrict__ v, int ldv,
+                                                                 const float* __restrict__ beta, int ldbeta,
+                                                                 const float* __restrict__ z, int ldz,
+                                                                 const float* __restrict__ dt_bias,
+                                                                 const float* __restrict__ a_log,
+                                                                 float* __restrict__ state, float* __restrict__ out,
+                                                                 int ldo, ScanShape sh) {
+  extern __shared__ float lds[];
+  constexpr int NP = LN * SLAB;  // a shared row in LDS, padded with zeros: entries past N take part as zeros
+  constexpr int TT = dch_tokens(NP, TH, LN);
+  constexpr int PER = (3 * TT * NP + TH - 1) / TH;
+  constexpr int cols = TH / LN;
+  constexpr int XPRE = (TT * cols + TH - 1) / TH;
+  constexpr int BUF = TT * (3 * NP + 2 * cols + 1);  // q, k, decays [TT][NP]; v, results [TT][cols]; beta [TT]
+  const int heads = sh.heads, P = sh.P, N = sh.N;
+  const int b = blockIdx.x / heads, h = blockIdx.x % heads, j = h / (heads / sh.groups);
+  const int tid = threadIdx.x, l = tid % LN, col = tid / LN, p0 = blockIdx.y * cols, p = p0 + col;
+  const bool live = p < P;
+  const long long r0 = sh.cu_rows[b], r1 = sh.cu_rows[b + 1];
+  float* sp = state + (((long long)sh.seq_slot[b] * heads + h) * P + (live ? p : 0)) * N;
+  float S[SLAB];
+#pragma unroll
+  for (int i = 0; i < SLAB; ++i) {
+    const int n = i * LN + l;
+    S[i] = (live && n < N) ? sp[n] : 0.f;
+  }
+  const float A = -expf(a_log[h]);
+  float pre[PER], xpre[XPRE], bpre = 0.f;
+  auto fetch = [&](long long c0, int nt) {  // the chunk's loads, into registers
+#pragma unroll
+    for (int jj = 0; jj < PER; ++jj) {
+      const int e = tid + jj * TH, which = e / (TT * NP), rem = e - which * (TT * NP), t = rem / NP, n = rem - t * NP;
+      float val = 0.f;
+      if (which < 3 && t < nt && n < N) {
+        const long long r = c0 + t;
+        val = which == 0 ? q[r * ldq + j * N + n] : which == 1 ? k[r * ldk + j * N + n] : z[r * ldz + h * N + n];
+      }
+      pre[jj] = val;
+    }
+#pragma unroll
+    for (int jj = 0; jj < XPRE; ++jj) {
+      const int e = tid + jj * TH, t = e / cols, c = e - t * cols;
+      xpre[jj] = (t < nt && p0 + c < P) ? v[(c0 + t) * ldv + h * P + p0 + c] : 0.f;
+    }
+    bpre = tid < nt ? beta[(c0 + tid) * ldbeta + h] : 0.f;
+  };
+  auto stash = [&](float* buf) {  // registers to LDS; the decay is made of its logit here
+#pragma unroll
+    for (int jj = 0; jj < PER; ++jj) {
+      const int e = tid + jj * TH, which = e / (TT * NP), n = e % NP;
+      if (which >= 3) continue;
+      float val = pre[jj];
+      if (which == 2) val = n < N ? expf(A * softplus_f(val + dt_bias[h * N + n])) : 0.f;
+      buf[e] = val;
+    }
+#pragma unroll
+    for (int jj = 0; jj < XPRE; ++jj) {
+      const int e = tid + jj * TH;
+      if (e < TT * cols) buf[3 * TT * NP + e] = xpre[jj];
+    }
+    if (tid < TT) buf[3 * TT * NP + 2 * TT * cols + tid] = sigmoid_f(bpre);
+  };
+  int cur = 0;
+  if (r1 > r0) {
+    fetch(r0, (int)min((long long)TT, r1 - r0));
+    stash(lds);
+  }
+  __syncthreads();
+  for (long long c0 = r0; c0 < r1; c0 += TT, cur ^= 1) {
+    const int nt = (int)min((long long)TT, r1 - c0);
+    const int next = (int)min((long long)TT, r1 - c0 - TT);
+    if (next > 0) fetch(c0 + TT, next);
+    float* buf = lds + cur * BUF;
+    const float *qs = buf, *ks = buf + TT * NP, *as = buf + 2 * TT * NP, *vs = buf + 3 * TT * NP;
+    const float* bs = buf + 3 * TT * NP + 2 * TT * cols;
+    float* os = buf + 3 * TT * NP + TT * cols;
+    struct Tok {  // (the next token's operands are read while this one is computed)
+      float q[SLAB], k[SLAB], a[SLAB], v, beta;
+    };
+    auto load = [&](Tok& x, int t) {
+      x.v = vs[t * cols + col], x.beta = bs[t];
+#pragma unroll
+      for (int i = 0; i < SLAB; ++i) {
+        const int n = t * NP + i * LN + l;
+        x.q[i] = qs[n], x.k[i] = ks[n], x.a[i] = as[n];
+      }
+    };
+    auto compute = [&](const Tok& x, int t) {
+      float sk = 0.f, sk1 = 0.f;  // (two chains, even and odd entries)
+#pragma unroll
+      for (int i = 0; i < SLAB; i += 2) {
+        S[i] *= x.a[i];
+        S[i + 1] *= x.a[i + 1];
+        sk = fmaf(S[i], x.k[i], sk);
+        sk1 = fmaf(S[i + 1], x.k[i + 1], sk1);
+      }
+      const float u = x.beta * (x.v - group_sum<LN>(sk + sk1));
+      float o = 0.f, o1 = 0.f;
+#pragma unroll
+      for (int i = 0; i < SLAB; i += 2) {
+        S[i] = fmaf(x.k[i], u, S[i]);
+        S[i + 1] = fmaf(x.k[i + 1], u, S[i + 1]);
+        o = fmaf(S[i], x.q[i], o);
+        o1 = fmaf(S[i + 1], x.q[i + 1], o1);
+      }
+      o = group_sum<LN>(o + o1);
+      if (l == 0) os[t * cols + col] = o;
+    };
+    Tok ta, tb;
+    load(ta, 0);
+#pragma unroll
+    for (int t = 0; t < TT; t += 2) {  // (unrolled: a token's places in LDS are constants)
+      if (t >= nt) break;
+      if (t + 1 < nt) load(tb, t + 1);
+      compute(ta, t);
+      if (t + 1 < nt) {
+        if (t + 2 < nt) load(ta, t + 2);
+        compute(tb, t + 1);
+      }
+    }
+    if (next > 0) stash(lds + (cur ^ 1) * BUF);
+    __syncthreads();
+    for (int e = tid; e < nt * cols; e += TH) {
+      const int t = e / cols, c = e - t * cols;
+      if (p0 + c < P) out[(c0 + t) * ldo + h * P + p0 + c] = os[e];
+    }
+  }
+  if (live) {
+#pragma unroll
+    for (int i = 0; i < SLAB; ++i) {
+      const int n = i * LN + l;
+      if (n < N) sp[n] = S[i];
+    }
+  }
+}
+
 // ---------------------------------------------------------------- norms after the scans
 // One workgroup a (row, group of `group` columns).  gate_first: v = y silu(z), out = v / rms(v) w;
-// else: out = y / rms(y) w silu(z).  w has `wlen` entries and repeats (one weight for all groups, or one a column).
+// else: out = y / rms(y) w silu(z).  `sigmoid_gate`: sigmoid(z) in the place of silu(z).  w has `wlen` entries and repeats (one weight for all groups, or one a column).
 template <typename T>
 __global__ void gated_rmsnorm_kernel(const float* __restrict__ y, int ldy, const float* __restrict__ z, int ldz,
                                      const float* __restrict__ w, int wlen, float eps, int group, T* __restrict__ out,
-                                     int ldo, int gate_first) {
+                                     int ldo, int gate_first, int sigmoid_gate) {
   __shared__ float red[16];
   const int r = blockIdx.y, c0 = blockIdx.x * group;
   const float* yr = y + (long long)r * ldy + c0;
   const float* zr = z + (long long)r * ldz + c0;
   float ss = 0.f;
   for (int c = threadIdx.x; c < group; c += blockDim.x) {
-    const float v = gate_first ? yr[c] * silu_f(zr[c]) : yr[c];
+    const float v = gate_first ? yr[c] * (sigmoid_gate ? sigmoid_f(zr[c]) : silu_f(zr[c])) : yr[c];
     ss = fmaf(v, v, ss);
   }
   const float inv = 1.f / sqrtf(block_sum(ss, red) / group + eps);
   for (int c = threadIdx.x; c < group; c += blockDim.x) {
-    const float gate = silu_f(zr[c]);
+    const float gate = sigmoid_gate ? sigmoid_f(zr[c]) : silu_f(zr[c]);
     const float v = gate_first ? yr[c] * gate * inv * w[(c0 + c) % wlen] : yr[c] * inv * w[(c0 + c) % wlen] * gate;
     store_as<T>(out + (long long)r * ldo + c0 + c, v);
   }
@@ -830,17 +987,17 @@ extern "C" int lq_add_scaled(float* x, const float* delta, int pieces, long long
 }
 
 extern "C" int lq_glu(const void* gu, int in_dtype, int ld, void* out, int out_dtype, int ldo, int rows, int I, int act,
-                      hipStream_t stream) {
-  LQ_REQUIRE(rows > 0 && I > 0 && ld >= 2 * I && ldo >= I, "glu: rows %d, inner %d, strides %d and %d", rows, I, ld, ldo);
+                      const float* bias, int tail, hipStream_t stream) {
+  LQ_REQUIRE(rows > 0 && I > 0 && ld >= 2 * I && tail >= 0 && ldo >= I + tail, "glu: rows %d, inner %d, strides %d and %d", rows, I, ld, ldo);
   LQ_REQUIRE(act >= ACT_SILU && act <= ACT_GELU_TANH, "glu: unknown activation %d", act);
   LQ_REQUIRE(rows <= 65535 * 64, "glu: too many rows");
   LQ_REQUIRE(gu && out, "glu: null pointer");
   for (int r0 = 0; r0 < rows; r0 += 65535) {
     const int nr = rows - r0 < 65535 ? rows - r0 : 65535;
-    dim3 grid(lq_ceil_div(I, 256), nr);
+    dim3 grid(lq_ceil_div(I + tail, 256), nr);
 #define LQ_GLU(TI, TO)                                                                                              \
   glu_kernel<TI, TO><<<grid, 256, 0, stream>>>((const TI*)gu + (long long)r0 * ld, ld, (TO*)out + (long long)r0 * ldo, \
-                                               ldo, I, act)
+                                               ldo, I, act, bias, tail)
     if (in_dtype == LQ_F32 && out_dtype == LQ_F32) LQ_GLU(float, float);
     else if (in_dtype == LQ_F32 && out_dtype == LQ_BF16) LQ_GLU(float, bf16_t);
     else if (in_dtype == LQ_BF16 && out_dtype == LQ_BF16) LQ_GLU(bf16_t, bf16_t);
@@ -953,13 +1110,15 @@ extern "C" int lq_ssd_scan(const float* x, int ldx, const float* Bm, int ldb, co
 // q and k [rows, kv_heads * Dk], v [rows, heads * P], beta and a [rows, heads] (raw), state [slots, heads, P, Dk],
 // out [rows, heads * P]
 // (q and k are made unit vectors in place)
+// `channel_decay`: a [rows, heads * Dk] and dt_bias [heads * Dk], a decay for every key channel of every head
 extern "C" int lq_delta_scan(float* q, int ldq, float* k, int ldk, const float* v, int ldv, const float* beta,
                              int ldbeta, const float* a, int lda, const float* dt_bias, const float* a_log, float* state,
                              float* out, int ldo, int heads, int kv_heads, int Dk, int P, float q_scale, float unit_eps,
-                             const int* seq_slot, const int* cu_rows, int batch, int rows, hipStream_t stream) {
+                             const int* seq_slot, const int* cu_rows, int batch, int rows, int channel_decay,
+                             hipStream_t stream) {
   LQ_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && Dk > 0 && P > 0 && batch > 0, "delta_scan: bad sizes");
   LQ_REQUIRE(ldq >= kv_heads * Dk && ldk >= kv_heads * Dk && ldv >= heads * P && ldo >= heads * P && ldbeta >= heads &&
-                 lda >= heads, "delta_scan: a row stride is smaller than its row");
+                 lda >= (channel_decay ? heads * Dk : heads), "delta_scan: a row stride is smaller than its row");
   LQ_REQUIRE(q && k && v && beta && a && dt_bias && a_log && state && out && seq_slot && cu_rows, "delta_scan: null pointer");
   ScanLaunch cfg;
   LQ_REQUIRE(scan_launch(Dk, P, (long long)batch * heads, cfg), "delta_scan: key size %d is too large", Dk);
@@ -968,6 +1127,18 @@ extern "C" int lq_delta_scan(float* q, int ldq, float* k, int ldk, const float* 
   LQ_CHECK_LAUNCH("delta_scan(unit vectors)");
   dim3 grid((unsigned)(batch * heads), lq_ceil_div(P, cfg.cols));
   ScanShape sh = {heads, kv_heads, P, Dk, seq_slot, cu_rows};
+  if (channel_decay) {
+    const int np = cfg.ln * cfg.slab;
+    const size_t lds = 2 * (size_t)dch_tokens(np, cfg.threads, cfg.ln) * (3 * np + 2 * cfg.cols + 1) * sizeof(float);
+    LQ_REQUIRE(lds <= 64 * 1024, "delta_scan: key size %d is too large", Dk);
+#define LQ_DELTA_CH(LN, SL, TH)                                                                                           \
+  delta_channel_scan_kernel<LN, SL, TH><<<grid, cfg.threads, lds, stream>>>(q, ldq, k, ldk, v, ldv, beta, ldbeta, a, lda, \
+                                                                            dt_bias, a_log, state, out, ldo, sh)
+    LQ_SCAN_LANES(LQ_DELTA_CH)
+#undef LQ_DELTA_CH
+    LQ_CHECK_LAUNCH("delta_scan(channel decay)");
+    return 0;
+  }
 #define LQ_DELTA(LN, SL, TH)                                                                                             \
   delta_scan_kernel<LN, SL, TH><<<grid, cfg.threads, cfg.lds, stream>>>(q, ldq, k, ldk, v, ldv, beta, ldbeta, a, lda,      \
                                                                     dt_bias, a_log, state, out, ldo, sh)
@@ -979,7 +1150,7 @@ extern "C" int lq_delta_scan(float* q, int ldq, float* k, int ldk, const float* 
 
 extern "C" int lq_gated_rmsnorm(const float* y, int ldy, const float* z, int ldz, const float* w, int wlen, float eps,
                                 int group, void* out, int out_dtype, int ldo, int rows, int n, int gate_first,
-                                hipStream_t stream) {
+                                int sigmoid_gate, hipStream_t stream) {
   LQ_REQUIRE(rows > 0 && n > 0 && group > 0 && n % group == 0, "gated_rmsnorm: %d columns in groups of %d", n, group);
   LQ_REQUIRE(wlen > 0 && (wlen == n || group % wlen == 0), "gated_rmsnorm: a weight of %d entries for groups of %d", wlen, group);
   LQ_REQUIRE(ldy >= n && ldz >= n && ldo >= n, "gated_rmsnorm: a row stride is smaller than its row");
@@ -990,10 +1161,10 @@ extern "C" int lq_gated_rmsnorm(const float* y, int ldy, const float* z, int ldz
     dim3 grid(n / group, nr);
     if (out_dtype == LQ_F32)
       gated_rmsnorm_kernel<float><<<grid, threads, 0, stream>>>(y + (long long)r0 * ldy, ldy, z + (long long)r0 * ldz, ldz, w,
-                                                               wlen, eps, group, (float*)out + (long long)r0 * ldo, ldo, gate_first);
+                                                               wlen, eps, group, (float*)out + (long long)r0 * ldo, ldo, gate_first, sigmoid_gate);
     else if (out_dtype == LQ_BF16)
       gated_rmsnorm_kernel<bf16_t><<<grid, threads, 0, stream>>>(y + (long long)r0 * ldy, ldy, z + (long long)r0 * ldz, ldz, w,
-                                                                wlen, eps, group, (bf16_t*)out + (long long)r0 * ldo, ldo, gate_first);
+                                                                wlen, eps, group, (bf16_t*)out + (long long)r0 * ldo, ldo, gate_first, sigmoid_gate);
     else
       LQ_REQUIRE(false, "gated_rmsnorm: unknown dtype %d", out_dtype);
   }

@@ -20,7 +20,7 @@ from .. import build as _build
 from .dry import query
 
 F32, BF16 = 0, 1
-ABI_VERSION = 7  # lq_abi_version() of the library these wrappers were written for
+ABI_VERSION = 8  # lq_abi_version() of the library these wrappers were written for
 _DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
 
 
@@ -779,15 +779,21 @@ class HipKernels:
         self._check(self.lib.lq_add_scaled(_ptr(x), _ptr(delta), c_int(pieces), c_longlong(stride), c_float(scale),
                                            c_longlong(x.numel()), self.stream))
 
-    def glu(self, gate_up: torch.Tensor, out: torch.Tensor, activation: str) -> None:
-        """out = act(gate) * up for gate_up [rows, 2 * inner] = [gate | up]; act: silu, relu or gelu_tanh."""
+    def glu(self, gate_up: torch.Tensor, out: torch.Tensor, activation: str, bias: Optional[torch.Tensor] = None,
+            tail: int = 0) -> None:
+        """out = act(gate) * up for gate_up [rows, 2 * inner] = [gate | up]; act: silu, relu or gelu_tanh.  `bias`
+        (float32 [2 * inner]) is added to gate and up first.  With `tail` out is [rows, inner + tail] and its last
+        columns become a one and then zeros (the next product's bias rides as one more column of its weight)."""
         rows, two, ld = self._mat(gate_up, "glu: gate_up")
-        ro, inner, ldo = self._mat(out, "glu: out")
-        if ro != rows or two != 2 * inner or activation not in self._ACTIVATIONS or activation == "none":
+        ro, wide, ldo = self._mat(out, "glu: out")
+        inner = wide - tail
+        if ro != rows or tail < 0 or two != 2 * inner or activation not in self._ACTIVATIONS or activation == "none":
             raise KernelLibraryError(f"glu: gate_up {tuple(gate_up.shape)}, out {tuple(out.shape)}, activation {activation!r}")
+        if bias is not None:
+            self._f32(bias, "glu: bias", 2 * inner)
         self._check(self.lib.lq_glu(_ptr(gate_up), c_int(_code(gate_up)), c_int(ld), _ptr(out), c_int(_code(out)),
                                     c_int(ldo), c_int(rows), c_int(inner), c_int(self._ACTIVATIONS[activation]),
-                                    self.stream))
+                                    _ptr(bias), c_int(tail), self.stream))
 
     def causal_conv(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], state: torch.Tensor,
                     out: torch.Tensor, row_pos: torch.Tensor, row_seq: torch.Tensor, seq_slot: torch.Tensor,
@@ -859,18 +865,21 @@ class HipKernels:
     def delta_scan(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, beta: torch.Tensor, a: torch.Tensor,
                    dt_bias: torch.Tensor, a_log: torch.Tensor, state: torch.Tensor, out: torch.Tensor, heads: int,
                    kv_heads: int, key_dim: int, value_dim: int, q_scale: float, unit_eps: float,
-                   seq_slot: torch.Tensor, cu_rows: torch.Tensor, batch: int) -> None:
+                   seq_slot: torch.Tensor, cu_rows: torch.Tensor, batch: int, channel_decay: bool = False) -> None:
         """The gated delta rule along every sequence of the step, token by token: q and k made unit vectors per
         head (x / sqrt(sum x^2 + unit_eps)), q times q_scale, beta = sigmoid(beta), g = exp(-exp(a_log)
         softplus(a + dt_bias)); S <- g S, u = beta (v - S^T k), S <- S + k u^T, out = S^T q.  state [slots, heads,
-        value_dim, key_dim].  All float32.  q and k are overwritten with their unit vectors."""
+        value_dim, key_dim].  All float32.  q and k are overwritten with their unit vectors.  The decay is one number
+        a head (a [rows, heads], dt_bias [heads]) or, with `channel_decay`, one for every key channel of every head
+        (a [rows, heads * key_dim], dt_bias [heads * key_dim]), multiplying the state's rows of that channel."""
         rows = q.shape[0]
+        n_decay = heads * key_dim if channel_decay else heads
         for t, what, cols in ((q, "q", kv_heads * key_dim), (k, "k", kv_heads * key_dim), (v, "v", heads * value_dim),
-                              (beta, "beta", heads), (a, "a", heads), (out, "out", heads * value_dim)):
+                              (beta, "beta", heads), (a, "a", n_decay), (out, "out", heads * value_dim)):
             self._f32(t, "delta_scan: " + what)
             if self._mat(t, "delta_scan: " + what)[:2] != (rows, cols):
                 raise KernelLibraryError(f"delta_scan: {what} must be [{rows}, {cols}], found {tuple(t.shape)}")
-        self._f32(dt_bias, "delta_scan: dt_bias", heads)
+        self._f32(dt_bias, "delta_scan: dt_bias", n_decay)
         self._f32(a_log, "delta_scan: a_log", heads)
         self._f32(state, "delta_scan: state")
         if state.dim() != 4 or tuple(state.shape[1:]) != (heads, value_dim, key_dim) or not state.is_contiguous():
@@ -883,13 +892,17 @@ class HipKernels:
                                            c_int(ld(a, "a")), _ptr(dt_bias), _ptr(a_log), _ptr(state), _ptr(out),
                                            c_int(ld(out, "out")), c_int(heads), c_int(kv_heads), c_int(key_dim),
                                            c_int(value_dim), c_float(q_scale), c_float(unit_eps), _ptr(seq_slot),
-                                           _ptr(cu_rows), c_int(batch), c_int(rows), self.stream))
+                                           _ptr(cu_rows), c_int(batch), c_int(rows), c_int(1 if channel_decay else 0),
+                                           self.stream))
 
     def gated_rmsnorm(self, y: torch.Tensor, z: torch.Tensor, weight: torch.Tensor, eps: float, group: int,
-                      out: torch.Tensor, gate_first: bool = True) -> None:
+                      out: torch.Tensor, gate_first: bool = True, gate: str = "silu") -> None:
         """RMS norm of y [rows, n] in parts of `group` columns, each by its own root mean square, with a gate
         silu(z): gate_first: (y silu(z)) normed, times weight; else y normed, times weight, times silu(z).  The
-        weight has n entries, or fewer that repeat (one weight for every part)."""
+        weight has n entries, or fewer that repeat (one weight for every part).  `gate` "sigmoid": sigmoid(z) in the
+        place of silu(z)."""
+        if gate not in ("silu", "sigmoid"):
+            raise KernelLibraryError(f"gated_rmsnorm: the gate is 'silu' or 'sigmoid', found {gate!r}")
         rows, n, ldy = self._mat(y, "gated_rmsnorm: y")
         rz, nz, ldz = self._mat(z, "gated_rmsnorm: z")
         ro, no, ldo = self._mat(out, "gated_rmsnorm: out")
@@ -901,7 +914,8 @@ class HipKernels:
         self._check(self.lib.lq_gated_rmsnorm(_ptr(y), c_int(ldy), _ptr(z), c_int(ldz), _ptr(weight),
                                               c_int(weight.numel()), c_float(eps), c_int(group), _ptr(out),
                                               c_int(_code(out)), c_int(ldo), c_int(rows), c_int(n),
-                                              c_int(1 if gate_first else 0), self.stream))
+                                              c_int(1 if gate_first else 0), c_int(1 if gate == "sigmoid" else 0),
+                                              self.stream))
 
     def rmsnorm_mean(self, stack: torch.Tensor, weights, eps: float, out: torch.Tensor) -> None:
         """out = mean over i of stack[i] / rms(stack[i]) * weights[i], row by row; stack [n, rows, width] float32."""
@@ -984,6 +998,67 @@ class HipKernels:
                                        c_int(1 if interleaved else 0), _ptr(freqs), c_float(magnitude), _ptr(row_pos),
                                        self.stream))
 
+    def rotary_qkv(self, src: torch.Tensor, q_out: torch.Tensor, k_out: torch.Tensor, v_out: torch.Tensor, heads: int,
+                   kv_heads: int, key_dim: int, value_dim: int, dims: int, interleaved: bool,
+                   freqs: Optional[torch.Tensor], magnitude: float, norm_eps: Optional[float],
+                   row_pos: torch.Tensor) -> None:
+        """src float32 [rows, (heads + kv_heads) key_dim + kv_heads value_dim] = [queries | keys | values] goes to
+        q_out, k_out and v_out in their dtype: of every query and key head the first `dims` entries rotated by
+        row_pos[r] * freqs (float64 [dims / 2]; pairing and magnitude as `rotary`), then, with `norm_eps` not None,
+        the head divided by its root mean square over key_dim (eps inside the root); values pass."""
+        rows, ns, lds = self._mat(src, "rotary_qkv: src")
+        rq, nq, ldq = self._mat(q_out, "rotary_qkv: q")
+        rk, nk, ldk = self._mat(k_out, "rotary_qkv: k")
+        rv, nv, ldv = self._mat(v_out, "rotary_qkv: v")
+        self._i32(row_pos, "row_pos", rows)
+        if src.dtype != torch.float32 or ns != (heads + kv_heads) * key_dim + kv_heads * value_dim \
+                or (rq, nq) != (rows, heads * key_dim) or (rk, nk) != (rows, kv_heads * key_dim) \
+                or (rv, nv) != (rows, kv_heads * value_dim) or not q_out.dtype == k_out.dtype == v_out.dtype:
+            raise KernelLibraryError("rotary_qkv: src float32 [rows, q | k | v], outputs of one dtype with their sizes")
+        if dims and (freqs is None or freqs.dtype != torch.float64 or not freqs.is_cuda or not freqs.is_contiguous()
+                     or freqs.numel() != dims // 2):
+            raise KernelLibraryError(f"rotary_qkv: {dims // 2} float64 frequencies on the GPU")
+        self._check(self.lib.lq_rotary_qkv(_ptr(src), c_int(lds), _ptr(q_out), c_int(ldq), _ptr(k_out), c_int(ldk),
+                                           _ptr(v_out), c_int(ldv), c_int(_code(q_out)), c_int(rows), c_int(heads),
+                                           c_int(kv_heads), c_int(key_dim), c_int(value_dim), c_int(dims),
+                                           c_int(1 if interleaved else 0), _ptr(freqs if dims else None),
+                                           c_float(magnitude), c_float(-1.0 if norm_eps is None else norm_eps),
+                                           _ptr(row_pos), self.stream))
+
+    def postnorm_residual(self, x: torch.Tensor, y: torch.Tensor, scales, weight: torch.Tensor, eps: float,
+                          extra: Optional[torch.Tensor] = None, next_weight: Optional[torch.Tensor] = None,
+                          next_eps: float = 0.0, h: Optional[torch.Tensor] = None) -> None:
+        """With y the sum of scales[i] * y[i] over a stack [n, rows, width] of 1 to 4 pieces (or y [rows, width] and
+        one scale): x += y / sqrt(mean(y^2) + eps) * weight; then x += extra, where given; then, where `h` is given,
+        h = x / sqrt(mean(x^2) + next_eps) * next_weight in the dtype of h.  x, y, extra float32."""
+        rows, width = x.shape
+        self._f32(x, "postnorm_residual: x", rows * width)
+        self._f32(y, "postnorm_residual: y")
+        pieces, stride = self._pieces(y, x, "postnorm_residual")
+        if len(scales) != pieces or not 1 <= pieces <= 4:
+            raise KernelLibraryError(f"postnorm_residual: {pieces} pieces and {len(scales)} scales (1 to 4 of each)")
+        self._f32(weight, "postnorm_residual: weight", width)
+        if extra is not None:
+            self._f32(extra, "postnorm_residual: extra", rows * width)
+        if (h is None) != (next_weight is None):
+            raise KernelLibraryError("postnorm_residual: the next norm's weight and its output come together")
+        if h is not None:
+            self._f32(next_weight, "postnorm_residual: next weight", width)
+            self._dev(h)
+            if tuple(h.shape) != (rows, width) or not h.is_contiguous():
+                raise KernelLibraryError("postnorm_residual: h must be dense and shaped like x")
+        sc = [float(v) for v in scales] + [0.0] * (4 - pieces)
+        self._check(self.lib.lq_postnorm_residual(_ptr(x), _ptr(y), c_int(pieces), c_longlong(stride), c_float(sc[0]),
+                                                  c_float(sc[1]), c_float(sc[2]), c_float(sc[3]), _ptr(weight),
+                                                  c_float(eps), _ptr(extra), _ptr(next_weight), c_float(next_eps),
+                                                  _ptr(h), c_int(_code(h) if h is not None else 0), c_int(rows),
+                                                  c_int(width), self.stream))
+
+    def scale(self, x: torch.Tensor, factor: float) -> None:
+        """x *= factor (dense float32)."""
+        self._f32(x, "scale: x", x.numel())
+        self._check(self.lib.lq_scale(_ptr(x), c_float(factor), c_longlong(x.numel()), self.stream))
+
     def linear_heads(self, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, heads: int, out_head_stride: int) -> None:
         """A product a head: out[r, h out_head_stride .. + N) = x[r, h K .. + K) . w[h]^T with w [heads, N, K]: one
         launch for bfloat16 operands with K in 16s, else a product a head."""
@@ -1048,20 +1123,30 @@ class HipKernels:
                                          c_int(max_rows if workspace is not None else 0), _ptr(workspace),
                                          c_longlong(0 if workspace is None else workspace.numel()), self.stream))
 
-    def moe_route(self, logits: torch.Tensor, route: torch.Tensor, top: int, renormalize: bool = False) -> None:
+    def moe_route(self, logits: torch.Tensor, route: torch.Tensor, top: int, renormalize: bool = False,
+                  correction: Optional[torch.Tensor] = None, groups: int = 0, keep: int = 0) -> None:
         """route[r, e] = sigmoid(logits[r, e]) for the `top` experts with the largest scores (the lower index on a
-        tie; divided by the chosen scores' sum with `renormalize`), -1 for the others.  float32."""
+        tie; divided by the chosen scores' sum with `renormalize`), -1 for the others.  float32.  With `correction`
+        (float32 [experts]) the choice goes by score + correction, the weights stay the scores.  With `groups` > 1
+        the experts form that many equal groups of neighbours and only experts of the `keep` groups whose two largest
+        choice scores sum highest can be chosen."""
         rows, experts, ldz = self._mat(logits, "moe_route: logits")
         self._f32(logits, "moe_route: logits")
         self._f32(route, "moe_route: route", rows * experts)
+        if correction is not None:
+            self._f32(correction, "moe_route: correction", experts)
         self._check(self.lib.lq_moe_route(_ptr(logits), c_int(ldz), _ptr(route), c_int(rows), c_int(experts), c_int(top),
-                                          c_int(1 if renormalize else 0), self.stream))
+                                          c_int(1 if renormalize else 0), _ptr(correction), c_int(groups), c_int(keep),
+                                          self.stream))
 
     def moe_glu(self, gu: torch.Tensor, route: torch.Tensor, out: torch.Tensor, experts: int, ff: int, limit: float,
-                weight_input: bool = True) -> None:
+                weight_input: bool = True, activation: str = "clamped_swish") -> None:
         """gu [rows, experts * 2 ff] float32 (every expert's gate then up), route [rows, experts]; out [rows,
         experts * ff]: for a chosen expert with weight w, g = min(w gate, limit), u = clamp(w up, -limit, limit),
-        y = g sigmoid(1.702 g) (u + 1) (with `weight_input` false w multiplies y instead); 0 for the others."""
+        y = g sigmoid(1.702 g) (u + 1) (with `weight_input` false w multiplies y instead); 0 for the others.
+        `activation` "silu": y = silu(gate) up, no clamps."""
+        if activation not in ("clamped_swish", "silu"):
+            raise KernelLibraryError(f"moe_glu: unknown activation {activation!r}")
         rows, ng, ldg = self._mat(gu, "moe_glu: gu")
         ro, no, ldo = self._mat(out, "moe_glu: out")
         self._f32(gu, "moe_glu: gu")
@@ -1070,7 +1155,8 @@ class HipKernels:
             raise KernelLibraryError("moe_glu: gu [rows, experts * 2 ff] and out [rows, experts * ff]")
         self._check(self.lib.lq_moe_glu(_ptr(gu), c_longlong(ldg), _ptr(route), _ptr(out), c_int(_code(out)),
                                         c_longlong(ldo), c_int(rows), c_int(experts), c_int(ff), c_float(limit),
-                                        c_int(1 if weight_input else 0), self.stream))
+                                        c_int(1 if weight_input else 0), c_int(1 if activation == "silu" else 0),
+                                        self.stream))
 
     def weight_rows(self, w, start: int, n: int):
         """Rows start .. start + n of a product weight as a weight of its own: a view of a dense one; of a packed

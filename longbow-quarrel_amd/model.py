@@ -10,7 +10,10 @@ The schedule is a list of `Run(layer, cache_of)`.  The same layer may appear
 more than once: it then runs again with the same weights, and every run has a
 cache of its own (its inputs differ, so its keys and values do).  `cache_of = j`
 lets a run read what run number j of the schedule (an earlier one) wrote instead
-of writing its own.
+of writing its own.  `add_input` adds the embedding's output (the stream as it was
+before the first run) to the stream right before the run: a model that runs a
+stretch of its layers several times feeds its input in again at the start of every
+pass but the first.
 """
 from __future__ import annotations
 
@@ -32,6 +35,7 @@ EMBEDDING_RUN = -1
 class Run:
     layer: int
     cache_of: Optional[int] = None  # read (never write) the cache of this earlier run of the schedule
+    add_input: bool = False  # the embedding's output is added to the stream right before this run
 
 
 @dataclass(frozen=True)
@@ -162,23 +166,40 @@ class DecoderModel:
         pending: Optional[torch.Tensor] = None
         if ctx.observe is not None:
             ctx.observe("embed", x, None)
+        x_in = None
+        if any(run.add_input for run in s.schedule):  # the stream as the embedding left it, kept for the step
+            x_in = ctx.ws.alloc(x.shape, torch.float32, keep=True)
+            kn.cast(x, x_in)
         for i, run in enumerate(s.schedule):
             ctx.ws.next_run()  # the buffers of the run before the last one are free again
             cache = caches.get(i if run.cache_of is None else run.cache_of)
             if cache is not None and run.cache_of is not None:
                 cache = cache.read_only()
             block = self.blocks[run.layer]
+            if run.add_input and not getattr(pending, "added_extra", False):
+                # the block's first norm adds it on its way, as it adds any pending delta
+                if hasattr(pending, "settle"):
+                    pending = pending.settle(x, ctx)
+                if pending is not None and not isinstance(pending, RowStats):
+                    kn.add(x, pending)
+                pending = x_in
+            more = {}
             if block.takes_next_norm:
                 if i + 1 < len(s.schedule):
                     after = self.blocks[s.schedule[i + 1].layer].first_norm
                 else:  # the final norm, where the head can take every row as it stands
                     after = self.final_norm if ctx.want_all and n_want == ctx.rows else None
-                pending = block.forward(x, pending, ctx, cache, next_norm=after)
-            else:
-                pending = block.forward(x, pending, ctx, cache)
+                more["next_norm"] = after
+            if getattr(block, "takes_next_extra", False) and i + 1 < len(s.schedule) and s.schedule[i + 1].add_input:
+                more["next_extra"] = x_in  # a block that can adds it itself, with its last kernel
+            pending = block.forward(x, pending, ctx, cache, **more)
             if ctx.observe is not None:
                 ctx.observe(f"run {i}", x, None if isinstance(pending, RowStats) or hasattr(pending, "settle")
                             else pending)
+        normed_ahead = None  # the last block has applied the final norm to every row already
+        if getattr(pending, "norm", None) is self.final_norm and getattr(pending, "normed", None) is not None \
+                and ctx.want_all and n_want == ctx.rows:
+            normed_ahead = pending.normed
         if hasattr(pending, "settle"):  # a pending object of a block's own kind adds itself to the stream
             pending = pending.settle(x, ctx)
         if n_want == 0:
@@ -192,7 +213,9 @@ class DecoderModel:
         folded = ctx.want_all and n_want == ctx.rows and isinstance(pending, RowStats) \
             and pending.norm is self.final_norm \
             and project_normed(kn, ctx, NormedRows(x, self.final_norm, pending), self.head, logits)
-        if not folded:
+        if normed_ahead is not None:
+            project(kn, ctx, normed_ahead, self.head, logits)
+        elif not folded:
             picked = ctx.ws.alloc((n_want, s.width), torch.float32)
             kn.gather_rows(x, want_rows, picked, delta=None if isinstance(pending, RowStats) else pending)
             normed = self.final_norm.forward(picked, ctx)

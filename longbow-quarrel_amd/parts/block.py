@@ -239,3 +239,109 @@ class OutputNormBlock(Block):
         if self.ffn is not None:
             h = self._add_normed(x, self._run(self.ffn, (h, ctx), ctx, x.shape[1]), self.ffn_norm, ctx)
         return RoundedStream(h) if h is not x else None
+
+
+class NormedAhead:
+    """What a `SandwichNormBlock` leaves pending: the stream x is up to date, and `normed` holds `norm` applied to it
+    (the norm that the stream meets next), made by the kernel that added the block's last result.  A reader whose
+    norm it is takes `normed`; anyone else has nothing to add (`settle`).  `added_extra`: the kernel also added what
+    the model wants added ahead of the next run."""
+
+    def __init__(self, normed: Optional[torch.Tensor], norm, added_extra: bool = False) -> None:
+        self.normed, self.norm, self.added_extra = normed, norm, added_extra
+
+    def settle(self, x: torch.Tensor, ctx: StepContext) -> None:
+        return None
+
+
+@BLOCKS.register("sandwich_norm")
+class SandwichNormBlock(Block):
+    """A norm ahead of every sublayer and one on its result: x += norm1b(mixer(norm1(x))); x += norm2b(ffn(norm2(x))).
+    All four are RMS norms.  One kernel takes a sublayer's result (the sum of its pieces, each with its scale: two
+    mixers side by side, routed experts beside a shared one), norms it, adds it to the 32-bit stream and applies the
+    norm that the stream meets next: the feed-forward's, or the next block's first.  The feed-forward may be absent
+    (`feed_forward=None`; its two norms then bind no tensors)."""
+
+    takes_next_norm = True
+    takes_next_extra = True  # forward(..., next_extra=t): t is added to the stream after the block's last result
+
+    def __init__(self, mixer: PartSpec, mixer_norm: PartSpec, mixer_out_norm: PartSpec,
+                 feed_forward: Optional[PartSpec] = None, ffn_norm: Optional[PartSpec] = None,
+                 ffn_out_norm: Optional[PartSpec] = None) -> None:
+        self.mixer = build_part(MIXERS, mixer)
+        self.mixer_norm = build_part(NORMS, mixer_norm)
+        self.mixer_out_norm = build_part(NORMS, mixer_out_norm)
+        self.ffn = build_part(FEED_FORWARDS, feed_forward) if feed_forward is not None else None
+        if self.ffn is not None and (ffn_norm is None or ffn_out_norm is None):
+            raise ValueError("a feed-forward needs the norm ahead of it and the norm of its result")
+        self.ffn_norm = build_part(NORMS, ffn_norm) if self.ffn is not None else None
+        self.ffn_out_norm = build_part(NORMS, ffn_out_norm) if self.ffn is not None else None
+        for norm in (self.mixer_norm, self.mixer_out_norm, self.ffn_norm, self.ffn_out_norm):
+            if norm is not None and not getattr(norm, "deferrable", False):
+                raise ValueError("the norms around the sublayers must be RMS norms")
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(p.graph_safe for p in self.parts())
+
+    @property
+    def first_norm(self):
+        return self.mixer_norm
+
+    def parts(self):
+        return tuple(p for p in (self.mixer_norm, self.mixer, self.mixer_out_norm, self.ffn_norm, self.ffn,
+                                 self.ffn_out_norm) if p is not None)
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [s for p in self.parts() for s in p.tensor_specs()]
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], env: BuildEnv) -> None:
+        super().bind(tensors, env)
+        for p in self.parts():
+            p.bind(tensors, env)
+
+    @staticmethod
+    def _result(part, args, ctx: StepContext, width: int):
+        """A sublayer's result as (pieces [n, rows, width] or [rows, width] in 32-bit, the pieces' scales)."""
+        in_pieces = getattr(part, "forward_pieces", None)
+        if in_pieces is not None:
+            return in_pieces(*args)
+        rows = args[0].shape[0]
+        if part.takes_out:
+            out = ctx.ws.alloc((rows, width), torch.float32)
+            part.forward(*args, out=out)
+            return out, (1.0,)
+        got = part.forward(*args)
+        if got.dtype == torch.float32 and got.is_contiguous() and (got.dim() == 2 or got.shape[0] <= 4):
+            return got, (1.0,) * (1 if got.dim() == 2 else got.shape[0])
+        out = ctx.ws.alloc((rows, width), torch.float32)
+        ParallelBlock._copy_into(ctx.kernels, got, out)
+        return out, (1.0,)
+
+    def forward(self, x: torch.Tensor, pending, ctx: StepContext, cache: Optional[LayerCache], next_norm=None,
+                next_extra=None):
+        kn = ctx.kernels
+        if isinstance(pending, NormedAhead) and pending.norm is self.mixer_norm and pending.normed is not None:
+            h = pending.normed
+        else:
+            if hasattr(pending, "settle"):
+                pending = pending.settle(x, ctx)
+            h = self.mixer_norm.forward(x, ctx, delta=None if isinstance(pending, RowStats) else pending)
+        y, scales = self._result(self.mixer, (h, ctx, cache), ctx, x.shape[1])
+        out_norm = self.mixer_out_norm
+        if self.ffn is not None:
+            h = ctx.ws.alloc(x.shape, ctx.dtype)
+            kn.postnorm_residual(x, y, scales, out_norm.weight, out_norm.eps, next_weight=self.ffn_norm.weight,
+                                 next_eps=self.ffn_norm.eps, h=h)
+            y, scales = self._result(self.ffn, (h, ctx), ctx, x.shape[1])
+            out_norm = self.ffn_out_norm
+        # whoever looks at the stream between blocks (`ctx.observe`) sees it as this block leaves it
+        extra = next_extra if ctx.observe is None else None
+        ahead = next_norm if getattr(next_norm, "deferrable", False) else None
+        h = ctx.ws.alloc(x.shape, ctx.dtype) if ahead is not None else None
+        kn.postnorm_residual(x, y, scales, out_norm.weight, out_norm.eps, extra=extra,
+                             next_weight=ahead.weight if ahead is not None else None,
+                             next_eps=ahead.eps if ahead is not None else 0.0, h=h)
+        if ahead is None and extra is None:
+            return None
+        return NormedAhead(h, ahead, added_extra=extra is not None)

@@ -8,7 +8,7 @@ from typing import Dict, List, Mapping, Optional
 
 import torch
 
-from .base import (FEED_FORWARDS, BuildEnv, FeedForward, NormedRows, StepContext, TensorSpec, product_weight, project,
+from .base import (FEED_FORWARDS, VECTOR32, BuildEnv, FeedForward, NormedRows, StepContext, TensorSpec, product_weight, project,
                    project_into, project_normed)
 
 
@@ -71,29 +71,38 @@ class SwiGLU(FeedForward):
 
 @FEED_FORWARDS.register("glu")
 class GatedLinearUnit(FeedForward):
-    """down(act(gate(h)) * up(h)) with a choice of `activation` ("relu", "silu", "gelu_tanh"); no biases.  gate
-    and up are one matrix product whose 32-bit result the activation kernel reads."""
+    """down(act(gate(h)) * up(h)) with a choice of `activation` ("relu", "silu", "gelu_tanh").  gate and up are one
+    matrix product whose 32-bit result the activation kernel reads.  With `bias` every projection has one
+    (`<name>.b`): the activation kernel adds gate's and up's; down's is one more column of its weight, which meets a
+    column of ones that the activation kernel leaves behind its result."""
 
     graph_safe = True
     ACTIVATIONS = ("silu", "relu", "gelu_tanh")
+    BIAS_TAIL = 8  # columns behind the activations: a one and zeros (a product's K stays a multiple of eight)
 
-    def __init__(self, width: int, inner: int, prefix: str, activation: str = "silu",
+    def __init__(self, width: int, inner: int, prefix: str, activation: str = "silu", bias: bool = False,
                  names: Optional[Mapping[str, str]] = None) -> None:
         if activation not in self.ACTIVATIONS:
             raise ValueError(f"unknown activation {activation!r}; known: {', '.join(self.ACTIVATIONS)}")
-        self.width, self.inner, self.activation = int(width), int(inner), activation
+        self.width, self.inner, self.activation, self.bias = int(width), int(inner), activation, bool(bias)
         n = {"gate": "gate", "up": "up", "down": "down"}
         n.update(names or {})
         self.names: Dict[str, str] = {key: f"{prefix}.{val}" for key, val in n.items()}
         self.w_gate_up: Optional[torch.Tensor] = None
         self.w_down: Optional[torch.Tensor] = None
+        self.b_gate_up: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> List[TensorSpec]:
-        return [
+        specs = [
             TensorSpec(self.names["gate"], (self.inner, self.width)),
             TensorSpec(self.names["up"], (self.inner, self.width)),
             TensorSpec(self.names["down"], (self.width, self.inner)),
         ]
+        if self.bias:
+            specs += [TensorSpec(self.names["gate"] + ".b", (self.inner,), kind=VECTOR32),
+                      TensorSpec(self.names["up"] + ".b", (self.inner,), kind=VECTOR32),
+                      TensorSpec(self.names["down"] + ".b", (self.width,))]  # (in the dtype of the matrix it joins)
+        return specs
 
     def bind(self, tensors: Mapping[str, torch.Tensor], env: BuildEnv) -> None:
         super().bind(tensors, env)
@@ -101,7 +110,12 @@ class GatedLinearUnit(FeedForward):
         if gate.dtype != up.dtype:
             raise ValueError(f"{self.names['gate']}: gate and up projections are stored in different dtypes")
         self.w_gate_up = product_weight(env, torch.cat([gate, up], dim=0))
-        self.w_down = product_weight(env, tensors[self.names["down"]])
+        down = tensors[self.names["down"]]
+        if self.bias:
+            self.b_gate_up = torch.cat([tensors[self.names["gate"] + ".b"], tensors[self.names["up"] + ".b"]]).contiguous()
+            b = tensors[self.names["down"] + ".b"].to(down.dtype)
+            down = torch.cat([down, b[:, None], down.new_zeros((self.width, self.BIAS_TAIL - 1))], dim=1)
+        self.w_down = product_weight(env, down)
 
     takes_out = True
 
@@ -110,8 +124,12 @@ class GatedLinearUnit(FeedForward):
         rows = h.shape[0]
         gu = ctx.ws.alloc((rows, 2 * self.inner), torch.float32)
         project(kn, ctx, h, self.w_gate_up, gu)
-        act = ctx.ws.alloc((rows, self.inner), ctx.dtype)
-        kn.glu(gu, act, self.activation)
+        if self.bias:
+            act = ctx.ws.alloc((rows, self.inner + self.BIAS_TAIL), self.w_down.dtype)
+            kn.glu(gu, act, self.activation, bias=self.b_gate_up, tail=self.BIAS_TAIL)
+        else:
+            act = ctx.ws.alloc((rows, self.inner), ctx.dtype)
+            kn.glu(gu, act, self.activation)
         if out is None:
             out = ctx.ws.alloc((rows, self.width), torch.float32)
         project(kn, ctx, act, self.w_down, out)
@@ -128,7 +146,14 @@ class MixtureOfExperts(FeedForward):
 
     Expert (`activation` "clamped_swish"): g = min(Wg h, limit), u = clamp(Wu h, -limit, limit),
     y = g sigmoid(1.702 g) (u + 1), result Wd y; no biases.  Wg (s h) = s (Wg h), so the weight is applied to the
-    32-bit results of the gate and up products, ahead of the clamps.
+    32-bit results of the gate and up products, ahead of the clamps.  `activation` "silu": y = silu(Wg h) (Wu h),
+    no clamps.
+
+    `correction`: a learned constant for every expert (`<prefix>.correction`) is added to the scores for the choice
+    alone; the weights stay the scores.  `groups` / `keep`: the experts form `groups` equal groups of neighbours, a
+    group's mark is the sum of its two largest choice scores, and only experts of the `keep` best groups can be
+    chosen.  `shared_inner`: one more expert of that inner size (`<prefix>.shared.*`, the same form) runs for every
+    token with weight one, and is added.
 
     How it runs.  The experts' gate and up matrices are one matrix [experts * 2 ff, width] and their down matrices
     one [width, experts * ff]: with the activations of the experts that a token did not choose set to zero, the down
@@ -144,18 +169,40 @@ class MixtureOfExperts(FeedForward):
     #: rows from which a step that is no decoding step is sorted by expert
     sort_from_rows = 256
 
-    def __init__(self, width: int, experts: int, top: int, inner: int, limit: float, prefix: str,
-                 weight_input: bool = True, renormalize: bool = False, names: Optional[Mapping[str, str]] = None) -> None:
+    ACTIVATIONS = ("clamped_swish", "silu")
+
+    def __init__(self, width: int, experts: int, top: int, inner: int, prefix: str, limit: float = 0.0,
+                 weight_input: bool = True, renormalize: bool = False, activation: str = "clamped_swish",
+                 correction: bool = False, groups: int = 0, keep: int = 0, shared_inner: int = 0,
+                 names: Optional[Mapping[str, str]] = None) -> None:
         self.width, self.experts, self.top, self.inner = int(width), int(experts), int(top), int(inner)
         self.limit, self.weight_input, self.renormalize = float(limit), bool(weight_input), bool(renormalize)
+        self.activation, self.correction = activation, bool(correction)
+        self.groups, self.keep, self.shared_inner = int(groups), int(keep), int(shared_inner)
+        if activation not in self.ACTIVATIONS:
+            raise ValueError(f"unknown activation {activation!r}; known: {', '.join(self.ACTIVATIONS)}")
+        if self.shared_inner and activation != "silu":
+            raise ValueError("a shared expert is built for the 'silu' activation only")
         if not 1 <= self.top <= self.experts:
             raise ValueError(f"{top} of {experts} experts cannot be chosen")
-        n = {"router": "router", "expert": "e{}", "gate": "gate", "up": "up", "down": "down"}
+        if self.groups > 1:
+            if self.experts % self.groups or not 1 <= self.keep <= self.groups or self.groups > 64:
+                raise ValueError(f"{experts} experts do not form {groups} equal groups of which {keep} are kept")
+            if self.keep * (self.experts // self.groups) < self.top:
+                raise ValueError(f"{keep} groups of {self.experts // self.groups} experts cannot give {top} experts")
+        else:
+            self.groups = self.keep = 0
+        n = {"router": "router", "expert": "e{}", "gate": "gate", "up": "up", "down": "down",
+             "correction": "correction", "shared": "shared"}
         n.update(names or {})
         self.prefix, self.n = prefix, n
+        self.w_correction: Optional[torch.Tensor] = None
 
     def _name(self, e: int, what: str) -> str:
         return f"{self.prefix}.{self.n['expert'].format(e)}.{self.n[what]}"
+
+    def _shared_name(self, what: str) -> str:
+        return f"{self.prefix}.{self.n['shared']}.{self.n[what]}"
 
     def tensor_specs(self) -> List[TensorSpec]:
         specs = []
@@ -163,51 +210,114 @@ class MixtureOfExperts(FeedForward):
             specs += [TensorSpec(self._name(e, "gate"), (self.inner, self.width)),
                       TensorSpec(self._name(e, "up"), (self.inner, self.width)),
                       TensorSpec(self._name(e, "down"), (self.width, self.inner))]
-        return specs + [TensorSpec(f"{self.prefix}.{self.n['router']}", (self.experts, self.width))]
+        specs.append(TensorSpec(f"{self.prefix}.{self.n['router']}", (self.experts, self.width)))
+        if self.correction:
+            specs.append(TensorSpec(f"{self.prefix}.{self.n['correction']}", (self.experts,), kind=VECTOR32))
+        if self.shared_inner:
+            specs += [TensorSpec(self._shared_name("gate"), (self.shared_inner, self.width)),
+                      TensorSpec(self._shared_name("up"), (self.shared_inner, self.width)),
+                      TensorSpec(self._shared_name("down"), (self.width, self.shared_inner))]
+        return specs
 
     def bind(self, tensors: Mapping[str, torch.Tensor], env: BuildEnv) -> None:
         super().bind(tensors, env)
         E = self.experts
         gu = [tensors[self._name(e, w)] for e in range(E) for w in ("gate", "up")]
         down = [tensors[self._name(e, "down")] for e in range(E)]
+        ffs = self.shared_inner
+        if ffs:  # the shared expert's rows and columns lie behind the routed experts'
+            gu += [tensors[self._shared_name(w)] for w in ("gate", "up")]
+            down.append(tensors[self._shared_name("down")])
         if len({m.dtype for m in gu + down}) != 1:
             raise ValueError(f"{self._name(0, 'gate')}: the experts' matrices are stored in different dtypes")
         # expert e's rows of the first matrix: [gate (ff) | up (ff)]; its columns of the second: e ff .. (e + 1) ff
         ff = self.inner
-        whole = torch.cat(gu, dim=0).contiguous()  # [E * 2 ff, width]
+        runs = [(e * 2 * ff, 2 * ff) for e in range(E)] + ([(E * 2 * ff, 2 * ffs)] if ffs else [])
+        whole = torch.cat(gu, dim=0).contiguous()  # [E * 2 ff (+ 2 ffs), width]
         self.w_gate_up = product_weight(env, whole)
         rows_of = getattr(env.kernels, "weight_rows", None)
         if self.w_gate_up is whole:
-            self.gate_up_of = [whole[e * 2 * ff : (e + 1) * 2 * ff] for e in range(E)]
+            self.gate_up_of = [whole[at : at + n] for at, n in runs]
         else:  # held in the products' own order: an expert's rows must be a weight in that order too
-            self.gate_up_of = [rows_of(self.w_gate_up, e * 2 * ff, 2 * ff) if rows_of else None for e in range(E)]
+            self.gate_up_of = [rows_of(self.w_gate_up, at, n) if rows_of else None for at, n in runs]
             if any(w is None for w in self.gate_up_of):
                 self.w_gate_up = whole
-                self.gate_up_of = [whole[e * 2 * ff : (e + 1) * 2 * ff] for e in range(E)]
+                self.gate_up_of = [whole[at : at + n] for at, n in runs]
         # the second matrix stays dense: an expert is a run of its columns, which only the dense order can give
-        self.w_down = torch.cat(down, dim=1).contiguous()  # [width, E * ff]
+        self.w_down = torch.cat(down, dim=1).contiguous()  # [width, E * ff (+ ffs)]
         self.down_of = [self.w_down[:, e * ff : (e + 1) * ff] for e in range(E)]
+        if ffs:
+            self.down_of.append(self.w_down[:, E * ff :])
+        if self.correction:
+            self.w_correction = tensors[f"{self.prefix}.{self.n['correction']}"].contiguous()
         # the router's product as it is stored: bfloat16 operands multiply exactly into 32-bit sums, and its result
         # (the logits) and everything after it are 32-bit
         self.w_router = tensors[f"{self.prefix}.{self.n['router']}"].contiguous()
 
-    def forward(self, h, ctx: StepContext, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-        kn = ctx.kernels
-        rows, E, ff = h.shape[0], self.experts, self.inner
+    def _route(self, h, ctx: StepContext) -> torch.Tensor:
+        kn, rows, E = ctx.kernels, h.shape[0], self.experts
         z = ctx.ws.alloc((rows, (E + 3) // 4 * 4), torch.float32)[:, :E]
         project(kn, ctx, h, self.w_router, z)
         route = ctx.ws.alloc((rows, E), torch.float32)  # the weight of a chosen expert, -1 for the others
-        kn.moe_route(z, route, self.top, self.renormalize)
+        more = {}
+        if self.correction:
+            more["correction"] = self.w_correction
+        if self.groups > 1:
+            more.update(groups=self.groups, keep=self.keep)
+        kn.moe_route(z, route, self.top, self.renormalize, **more)
+        return route
+
+    def _sorts(self, rows: int, ctx: StepContext) -> bool:
+        return rows >= self.sort_from_rows and not ctx.decode and not ctx.dry and self.experts > self.top \
+            and getattr(ctx.kernels, "moe_sort", None) is not None
+
+    def _unit(self, gu, act, ctx: StepContext) -> None:
+        """The shared expert's activation (weight one, no routing)."""
+        ctx.kernels.glu(gu, act, "silu")
+
+    def forward_pieces(self, h, ctx: StepContext):
+        """The result in pieces [n, rows, width] that the caller adds: the routed experts' sum, and the shared
+        expert's result where a step's rows were sorted by expert (otherwise one product adds both)."""
+        rows = h.shape[0]
+        if not (self.shared_inner and self._sorts(rows, ctx)):
+            out = ctx.ws.alloc((1, rows, self.width), torch.float32)
+            self.forward(h, ctx, out=out[0])
+            return out, (1.0,)
+        out = ctx.ws.alloc((2, rows, self.width), torch.float32)
+        self._sorted(h, self._route(h, ctx), out[0], ctx)
+        self._shared(h, out[1], ctx)
+        return out, (1.0, 1.0)
+
+    def _shared(self, h, out, ctx: StepContext) -> None:
+        kn, rows, ffs = ctx.kernels, h.shape[0], self.shared_inner
+        gu = ctx.ws.alloc((rows, 2 * ffs), torch.float32)
+        project(kn, ctx, h, self.gate_up_of[-1], gu)
+        act = ctx.ws.alloc((rows, ffs), ctx.dtype)
+        self._unit(gu, act, ctx)
+        project(kn, ctx, act, self.down_of[-1], out)
+
+    def forward(self, h, ctx: StepContext, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        kn = ctx.kernels
+        rows, E, ff, ffs = h.shape[0], self.experts, self.inner, self.shared_inner
+        route = self._route(h, ctx)
         if out is None:
             out = ctx.ws.alloc((rows, self.width), torch.float32)
-        if rows >= self.sort_from_rows and not ctx.decode and not ctx.dry and E > self.top \
-                and getattr(kn, "moe_sort", None) is not None:
+        if self._sorts(rows, ctx):
             self._sorted(h, route, out, ctx)
+            if ffs:
+                extra = ctx.ws.alloc((rows, self.width), torch.float32)
+                self._shared(h, extra, ctx)
+                kn.add(out, extra)
             return out
-        gu = ctx.ws.alloc((rows, E * 2 * ff), torch.float32)
+        # every row through all experts' columns (and the shared expert's behind them): the activations of the
+        # experts that a row did not choose are zeros, so the second product adds the chosen ones and the shared one
+        gu = ctx.ws.alloc((rows, E * 2 * ff + 2 * ffs), torch.float32)
         project(kn, ctx, h, self.w_gate_up, gu)
-        act = ctx.ws.alloc((rows, E * ff), ctx.dtype)
-        kn.moe_glu(gu, route, act, E, ff, self.limit, self.weight_input)
+        act = ctx.ws.alloc((rows, E * ff + ffs), ctx.dtype)
+        more = {"activation": self.activation} if self.activation != "clamped_swish" else {}
+        kn.moe_glu(gu[:, : E * 2 * ff], route, act[:, : E * ff], E, ff, self.limit, self.weight_input, **more)
+        if ffs:
+            self._unit(gu[:, E * 2 * ff :], act[:, E * ff :], ctx)
         project(kn, ctx, act, self.w_down, out)
         return out
 
@@ -235,7 +345,8 @@ class MixtureOfExperts(FeedForward):
                 project(kn, ctx, hs[at : at + n], self.gate_up_of[e], gu[at : at + n])
                 at += n
         act = ctx.ws.alloc((pairs, ff), ctx.dtype)
-        kn.moe_glu(gu[:total], weight[:total], act[:total], 1, ff, self.limit, self.weight_input)
+        more = {"activation": self.activation} if self.activation != "clamped_swish" else {}
+        kn.moe_glu(gu[:total], weight[:total], act[:total], 1, ff, self.limit, self.weight_input, **more)
         ys = ctx.ws.alloc((pairs, self.width), torch.float32)
         at = 0
         for e, n in enumerate(n_of):

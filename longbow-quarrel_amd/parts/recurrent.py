@@ -134,23 +134,40 @@ class GatedDelta(_Recurrent):
         S <- g S;   u = beta (v - S^T k);   S <- S + k u^T;   o = S^T q.
 
     Each head's o is divided by its root mean square, multiplied by a weight that the heads share and by
-    silu of one more projection of the input; then the output projection."""
+    silu of one more projection of the input; then the output projection.
+
+    `decay="channel"`: one decay for every key channel of every head, g = exp(-exp(A_log_h) softplus(W2 (W1 h) +
+    dt_bias)) with dt_bias [heads * key_dim] and the two matrices a bottleneck of `decay_rank` columns; S <- diag(g) S
+    multiplies the state's rows of a key channel.  `gate="sigmoid"`: the sigmoid of the gate's projection in the
+    place of silu; `gate_rank`: that projection through a bottleneck of so many columns (two matrices)."""
 
     UNIT_EPS = 1e-6
 
     def __init__(self, width: int, heads: int, kv_heads: int, key_dim: int, value_dim: int, conv: int, eps: float,
-                 prefix: str, names: Optional[Mapping[str, str]] = None) -> None:
+                 prefix: str, decay: str = "head", decay_rank: Optional[int] = None, gate: str = "silu",
+                 gate_rank: Optional[int] = None, names: Optional[Mapping[str, str]] = None) -> None:
         if heads % kv_heads != 0:
             raise ValueError(f"{heads} heads cannot share {kv_heads} q/k heads evenly")
+        if decay not in ("head", "channel") or gate not in ("silu", "sigmoid"):
+            raise ValueError(f"the decay is 'head' or 'channel' (found {decay!r}), the gate 'silu' or 'sigmoid' ({gate!r})")
+        if decay == "channel" and (decay_rank is None or int(decay_rank) < 1):
+            raise ValueError("a decay for every key channel comes through a bottleneck: its rank is needed")
+        if gate_rank is not None and int(gate_rank) < 1:
+            raise ValueError("the gate's bottleneck needs a rank of at least one")
         self.width, self.heads, self.kv_heads = int(width), int(heads), int(kv_heads)
         self.key_dim, self.value_dim, self.taps, self.eps = int(key_dim), int(value_dim), int(conv), float(eps)
         if self.taps < 1:
             raise ValueError("the convolution needs at least one tap")
+        self.channel_decay, self.gate_act = decay == "channel", gate
+        self.decay_rank = int(decay_rank) if self.channel_decay else 0
+        self.gate_rank = int(gate_rank) if gate_rank is not None else 0
         self.qk_width = self.kv_heads * self.key_dim
         self.v_width = self.heads * self.value_dim
         self.conv_channels = 2 * self.qk_width + self.v_width
+        self.n_decay = self.heads * self.key_dim if self.channel_decay else self.heads
         n = {"q": "q", "k": "k", "v": "v", "q_conv": "q.conv", "k_conv": "k.conv", "v_conv": "v.conv", "beta": "b",
-             "a": "a", "A_log": "A_log", "dt_bias": "dt_bias", "norm": "norm", "gate": "g", "o": "o"}
+             "a": "a", "a1": "a1", "a2": "a2", "A_log": "A_log", "dt_bias": "dt_bias", "norm": "norm", "gate": "g",
+             "g1": "g1", "g2": "g2", "o": "o"}
         n.update(names or {})
         self.names: Dict[str, str] = {key: f"{prefix}.{val}" for key, val in n.items()}
 
@@ -166,19 +183,39 @@ class GatedDelta(_Recurrent):
             TensorSpec(nm["beta"], (self.heads, self.width)),
             TensorSpec(nm["A_log"], (self.heads,), kind=VECTOR32),
             TensorSpec(nm["norm"], (self.value_dim,), kind=VECTOR32, init="around_one"),
-            TensorSpec(nm["a"], (self.heads, self.width)),
-            TensorSpec(nm["dt_bias"], (self.heads,), kind=VECTOR32),
-            TensorSpec(nm["gate"], (self.v_width, self.width)),
+            *([TensorSpec(nm["a1"], (self.decay_rank, self.width)), TensorSpec(nm["a2"], (self.n_decay, self.decay_rank))]
+              if self.channel_decay else [TensorSpec(nm["a"], (self.heads, self.width))]),
+            TensorSpec(nm["dt_bias"], (self.n_decay,), kind=VECTOR32),
+            *([TensorSpec(nm["g1"], (self.gate_rank, self.width)), TensorSpec(nm["g2"], (self.v_width, self.gate_rank))]
+              if self.gate_rank else [TensorSpec(nm["gate"], (self.v_width, self.width))]),
             TensorSpec(nm["o"], (self.width, self.v_width)),
         ]
 
     def bind(self, tensors: Mapping[str, torch.Tensor], env: BuildEnv) -> None:
         super().bind(tensors, env)
         nm = self.names
-        mats = [tensors[nm[k]] for k in ("q", "k", "v", "beta", "a", "gate")]
+        # one product of the input for everything that is read in 32-bit: [q | k | v | beta (| a) (| gate)]
+        whole = ["q", "k", "v", "beta"] + ([] if self.channel_decay else ["a"]) + ([] if self.gate_rank else ["gate"])
+        low = (["a1"] if self.channel_decay else []) + (["g1"] if self.gate_rank else [])
+        mats = [tensors[nm[k]] for k in whole + low]
         if len({m.dtype for m in mats}) != 1:
             raise ValueError(f"{nm['q']}: the projections of one input are stored in different dtypes")
-        self.w_in = product_weight(env, torch.cat(mats, dim=0))  # [q | k | v | beta | a | gate]
+        self.w_in = product_weight(env, torch.cat(mats[: len(whole)], dim=0))
+        # the bottlenecks' first matrices are one product of their own: its result feeds the second matrices in the
+        # run's dtype; each bottleneck's columns start on a multiple of eight
+        self.w_low, self.low_at, at = None, {}, 0
+        if low:
+            padded = []
+            for key in low:
+                m = tensors[nm[key]]
+                self.low_at[key] = at
+                pad = (-m.shape[0]) % 8
+                padded += [m] + ([m.new_zeros((pad, m.shape[1]))] if pad else [])
+                at += m.shape[0] + pad
+            self.w_low = product_weight(env, torch.cat(padded, dim=0))
+        self.low_width = at
+        self.w_a2 = product_weight(env, tensors[nm["a2"]]) if self.channel_decay else None
+        self.w_g2 = product_weight(env, tensors[nm["g2"]]) if self.gate_rank else None
         self.w_o = product_weight(env, tensors[nm["o"]])
         self.conv_w = torch.cat([tensors[nm[k]] for k in ("q_conv", "k_conv", "v_conv")], dim=0).contiguous()
         self.a_log, self.dt_bias, self.norm_w = (tensors[nm[k]].contiguous() for k in ("A_log", "dt_bias", "norm"))
@@ -192,19 +229,34 @@ class GatedDelta(_Recurrent):
         state, conv_state = self._states(cache)
         rows = h.shape[0]
         cc, nh = self.conv_channels, self.heads
-        total = cc + 2 * nh + self.v_width
+        n_a = 0 if self.channel_decay else nh
+        total = cc + nh + n_a + (0 if self.gate_rank else self.v_width)
         u = ctx.ws.alloc((rows, _round4(total)), torch.float32)[:, :total]
         project(kn, ctx, h, self.w_in, u)
+        decay, gate = u[:, cc + nh : cc + nh + n_a], u[:, cc + nh + n_a :]
+        if self.w_low is not None:
+            low = ctx.ws.alloc((rows, self.low_width), self.w_low.dtype)
+            project(kn, ctx, h, self.w_low, low)
+            if self.channel_decay:
+                at = self.low_at["a1"]
+                decay = ctx.ws.alloc((rows, self.n_decay), torch.float32)
+                project(kn, ctx, low[:, at : at + self.decay_rank], self.w_a2, decay)
+            if self.gate_rank:
+                at = self.low_at["g1"]
+                gate = ctx.ws.alloc((rows, self.v_width), torch.float32)
+                project(kn, ctx, low[:, at : at + self.gate_rank], self.w_g2, gate)
         qkv = ctx.ws.alloc((rows, _round4(cc)), torch.float32)[:, :cc]
         kn.causal_conv(u[:, :cc], self.conv_w, None, conv_state, qkv, ctx.row_pos, ctx.row_seq, ctx.seq_slot,
                        ctx.seq_start, ctx.seq_len, ctx.cu_rows, ctx.batch, activation="silu")
         o = ctx.ws.alloc((rows, self.v_width), torch.float32)
+        more = {"channel_decay": True} if self.channel_decay else {}
         kn.delta_scan(qkv[:, : self.qk_width], qkv[:, self.qk_width : 2 * self.qk_width], qkv[:, 2 * self.qk_width :],
-                      u[:, cc : cc + nh], u[:, cc + nh : cc + 2 * nh], self.dt_bias, self.a_log, state, o, self.heads,
+                      u[:, cc : cc + nh], decay, self.dt_bias, self.a_log, state, o, self.heads,
                       self.kv_heads, self.key_dim, self.value_dim, self.key_dim ** -0.5, self.UNIT_EPS,
-                      ctx.seq_slot, ctx.cu_rows, ctx.batch)
+                      ctx.seq_slot, ctx.cu_rows, ctx.batch, **more)
         normed = ctx.ws.alloc((rows, self.v_width), ctx.dtype)
-        kn.gated_rmsnorm(o, u[:, cc + 2 * nh :], self.norm_w, self.eps, self.value_dim, normed, gate_first=False)
+        more = {"gate": "sigmoid"} if self.gate_act == "sigmoid" else {}
+        kn.gated_rmsnorm(o, gate, self.norm_w, self.eps, self.value_dim, normed, gate_first=False, **more)
         if out is None:
             out = ctx.ws.alloc((rows, self.width), torch.float32)
         project(kn, ctx, normed, self.w_o, out)
@@ -214,16 +266,23 @@ class GatedDelta(_Recurrent):
 @MIXERS.register("side_by_side")
 class SideBySide(Mixer):
     """Several mixers that read the same input; the result is the mean of their outputs, each first divided
-    by its root mean square over the width and multiplied by a weight of its own (`out_names`)."""
+    by its root mean square over the width and multiplied by a weight of its own (`out_names`).  With `weights`
+    (a constant for each mixer) instead: the weighted sum of the outputs as they are, sum_i weights[i] * mixer_i(h);
+    a block that takes a result in pieces gets the outputs and the constants (`forward_pieces`)."""
 
     takes_out = True
 
-    def __init__(self, width: int, eps: float, sides, out_names) -> None:
+    def __init__(self, width: int, eps: float, sides, out_names=(), weights=None) -> None:
         self.width, self.eps = int(width), float(eps)
         self.sides = [MIXERS.get(s.kind)(**dict(s.params)) for s in sides]
         self.out_names = list(out_names)
-        if len(self.sides) != len(self.out_names) or not 1 <= len(self.sides) <= 4:
-            raise ValueError("one to four mixers side by side, each with the name of its output weight")
+        self.weights = None if weights is None else tuple(float(w) for w in weights)
+        if not 1 <= len(self.sides) <= 4:
+            raise ValueError("one to four mixers side by side")
+        if self.weights is None and len(self.sides) != len(self.out_names):
+            raise ValueError("mixers side by side: each with the name of its output weight, or a constant for each")
+        if self.weights is not None and (len(self.weights) != len(self.sides) or self.out_names):
+            raise ValueError("mixers side by side: a constant for each mixer, and then no output weights")
         self.out_w: List[torch.Tensor] = []
 
     @property
@@ -249,7 +308,7 @@ class SideBySide(Mixer):
     def lengths_uneven(self, kernels, lengths) -> bool:
         return any(s.lengths_uneven(kernels, lengths) for s in self.sides)
 
-    def forward(self, h: torch.Tensor, ctx: StepContext, cache, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    def _results(self, h: torch.Tensor, ctx: StepContext, cache) -> torch.Tensor:
         if not isinstance(cache, MultiCache) or len(cache.parts) != len(self.sides):
             raise RuntimeError("mixers side by side need a cache for each side")
         rows = h.shape[0]
@@ -260,9 +319,25 @@ class SideBySide(Mixer):
                 side.forward(h, ctx, part, out=results[i])
             else:
                 ctx.kernels.cast(side.forward(h, ctx, part), results[i])
+        return results
+
+    def forward_pieces(self, h: torch.Tensor, ctx: StepContext, cache):
+        """The mixers' outputs [n, rows, width] and the constants their sum is weighted with (a weighted sum only)."""
+        if self.weights is None:
+            return self.forward(h, ctx, cache), (1.0,)
+        return self._results(h, ctx, cache), self.weights
+
+    def forward(self, h: torch.Tensor, ctx: StepContext, cache, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        results = self._results(h, ctx, cache)
         if out is None:
-            out = ctx.ws.alloc((rows, self.width), torch.float32)
-        ctx.kernels.rmsnorm_mean(results, self.out_w, self.eps, out)
+            out = ctx.ws.alloc((h.shape[0], self.width), torch.float32)
+        if self.weights is None:
+            ctx.kernels.rmsnorm_mean(results, self.out_w, self.eps, out)
+            return out
+        ctx.kernels.cast(results[0], out)
+        ctx.kernels.scale(out, self.weights[0])
+        for piece, weight in zip(results[1:], self.weights[1:]):
+            ctx.kernels.add_scaled(out, piece, weight)
         return out
 
 

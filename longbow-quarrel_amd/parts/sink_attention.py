@@ -10,6 +10,12 @@ sigmoid of one more projection of h, a number per head.  Scores, probabilities a
 32-bit whatever the run's dtype.  A position encoding is optional (`position=None`: positions do not enter
 the scores).
 
+`rotary` (a mapping: `dims`, `base`, optionally `scaling` as `rope.rotary_frequencies` takes it and `pairing`,
+"interleaved" or "half") rotates the first `dims` entries of every query and key head by the position, the rest
+pass; `qk_norm_eps` then divides every query and key head by its root mean square over key_dim (no weight).  Both
+are taken in 32-bit on the product's 32-bit result, by one kernel that also leaves q, k and v in the dtype of the
+cache.
+
 All projections of h are one matrix product ([q | k | v | gate]).
 """
 from __future__ import annotations
@@ -20,6 +26,7 @@ import torch
 
 from .base import (MIXERS, POSITION_ENCODINGS, BuildEnv, KVNeed, LayerCache, Mixer, PartSpec, StepContext,
                    TensorSpec, build_part, product_weight, project)
+from .rope import rotary_frequencies, rotary_magnitude
 
 
 def split_scratch(ctx: StepContext, dtype, heads: int, kv_heads: int, key_dim: int, value_dim: int, block_size: int,
@@ -39,9 +46,28 @@ class SinkWindowAttention(Mixer):
 
     def __init__(self, width: int, heads: int, kv_heads: int, key_dim: int, value_dim: int, scale: float,
                  prefix: str, window: int = 0, keep_first: int = 0, sink: bool = True, head_gate: bool = False,
-                 position: Optional[PartSpec] = None, names: Optional[Mapping[str, str]] = None) -> None:
+                 position: Optional[PartSpec] = None, rotary: Optional[Mapping] = None,
+                 qk_norm_eps: Optional[float] = None, names: Optional[Mapping[str, str]] = None) -> None:
         if heads % kv_heads != 0:
             raise ValueError(f"{heads} heads cannot share {kv_heads} kv heads evenly")
+        self.rot_dims, self.rot_interleaved, self.rot_magnitude, self.freq_table = 0, False, 1.0, []
+        if rotary is not None:
+            if position is not None:
+                raise ValueError("a position encoding part or the `rotary` parameters, not both")
+            self.rot_dims = int(rotary["dims"])
+            pairing = rotary.get("pairing", "interleaved")
+            if pairing not in ("half", "interleaved"):
+                raise ValueError(f"rotary pairing {pairing!r} is not known (known: 'half', 'interleaved')")
+            if self.rot_dims % 2 or not 2 <= self.rot_dims <= int(key_dim):
+                raise ValueError(f"{self.rot_dims} rotated entries do not fit a head of {key_dim}")
+            scaling = dict(rotary["scaling"]) if rotary.get("scaling") else None
+            self.rot_interleaved = pairing == "interleaved"
+            self.freq_table = rotary_frequencies(self.rot_dims, float(rotary["base"]), scaling)
+            self.rot_magnitude = rotary_magnitude(scaling)
+        self.qk_norm_eps = None if qk_norm_eps is None else float(qk_norm_eps)
+        self.prepared = rotary is not None or qk_norm_eps is not None  # q, k and v pass the kernel named above
+        if self.prepared and head_gate:
+            raise ValueError("a gate per head and a rotation or norm of q and k are not combined")
         if window < 0 or keep_first < 0:
             raise ValueError("window and keep_first must not be negative")
         self.width, self.heads, self.kv_heads = int(width), int(heads), int(kv_heads)
@@ -83,6 +109,7 @@ class SinkWindowAttention(Mixer):
         self.w_o = product_weight(env, tensors[self.names["o"]])
         if self.position is not None:
             self.position.bind(tensors, env)
+        self.freqs = torch.tensor(self.freq_table, dtype=torch.float64, device=env.device) if self.rot_dims else None
 
     def cache_need(self) -> KVNeed:
         # a window that keeps first tokens still gives its middle blocks back
@@ -96,15 +123,26 @@ class SinkWindowAttention(Mixer):
         rows = h.shape[0]
         total = self.q_width + self.k_width + self.v_width + (self.heads if self.head_gate else 0)
         total_padded = (total + 3) // 4 * 4  # rows of the product start on 16 bytes
-        # q, k and v in the run's dtype (what the cache holds); the gate's logits ride in the same product
-        proj = ctx.ws.alloc((rows, total_padded), ctx.dtype)[:, :total]
-        project(kn, ctx, h, self.w_in, proj)
-        q = proj[:, : self.q_width]
-        k = proj[:, self.q_width : self.q_width + self.k_width]
-        v = proj[:, self.q_width + self.k_width : self.q_width + self.k_width + self.v_width]
-        gate = proj[:, self.q_width + self.k_width + self.v_width :] if self.head_gate else None
-        if self.position is not None:
-            self.position.apply(q, k, ctx)
+        if self.prepared:
+            # the product's 32-bit result is rotated and normed in 32-bit, then rounded to what the cache holds
+            proj = ctx.ws.alloc((rows, total_padded), torch.float32)[:, :total]
+            project(kn, ctx, h, self.w_in, proj)
+            q = ctx.ws.alloc((rows, self.q_width), ctx.dtype)
+            k = ctx.ws.alloc((rows, self.k_width), ctx.dtype)
+            v = ctx.ws.alloc((rows, self.v_width), ctx.dtype)
+            gate = None
+            kn.rotary_qkv(proj, q, k, v, self.heads, self.kv_heads, self.key_dim, self.value_dim, self.rot_dims,
+                          self.rot_interleaved, self.freqs, self.rot_magnitude, self.qk_norm_eps, ctx.row_pos)
+        else:
+            # q, k and v in the run's dtype (what the cache holds); the gate's logits ride in the same product
+            proj = ctx.ws.alloc((rows, total_padded), ctx.dtype)[:, :total]
+            project(kn, ctx, h, self.w_in, proj)
+            q = proj[:, : self.q_width]
+            k = proj[:, self.q_width : self.q_width + self.k_width]
+            v = proj[:, self.q_width + self.k_width : self.q_width + self.k_width + self.v_width]
+            gate = proj[:, self.q_width + self.k_width + self.v_width :] if self.head_gate else None
+            if self.position is not None:
+                self.position.apply(q, k, ctx)
         if cache.write:
             kn.kv_store(k, v, self.kv_heads, self.key_dim, self.value_dim, ctx.row_pos, ctx.row_seq, ctx.seq_slot,
                         cache.block_table, cache.k, cache.v, cache.block_size)

@@ -139,9 +139,11 @@ class CpuKernels:
     def add_scaled(self, x, delta, scale):
         x += self._whole(delta, x) * scale
 
-    def glu(self, gate_up, out, activation):
-        inner = out.shape[1]
+    def glu(self, gate_up, out, activation, bias=None, tail=0):
+        inner = out.shape[1] - tail
         g, u = gate_up[:, :inner].float(), gate_up[:, inner:].float()
+        if bias is not None:
+            g, u = g + bias[:inner], u + bias[inner:]
         if activation == "relu":
             a = torch.clamp(g, min=0)
         elif activation == "silu":
@@ -150,7 +152,10 @@ class CpuKernels:
             a = 0.5 * g * (1 + torch.tanh(math.sqrt(2 / math.pi) * (g + 0.044715 * g * g * g)))
         else:
             raise ValueError(activation)
-        out.copy_((a * u).to(out.dtype))
+        out[:, :inner] = (a * u).to(out.dtype)
+        if tail:
+            out[:, inner:] = 0
+            out[:, inner] = 1
 
     def kv_store(self, k, v, kv_heads, key_dim, value_dim, row_pos, row_seq, seq_slot, block_table, kcache, vcache,
                  block_size):
@@ -213,7 +218,7 @@ class CpuKernels:
                 y[r] = ((s * cr[:, None, :]).sum(-1) + d_skip[:, None] * xr).reshape(-1)
 
     def delta_scan(self, q, k, v, beta, a, dt_bias, a_log, state, out, heads, kv_heads, key_dim, value_dim, q_scale,
-                   unit_eps, seq_slot, cu_rows, batch):
+                   unit_eps, seq_slot, cu_rows, batch, channel_decay=False):
         rep = heads // kv_heads
         for b in range(batch):
             r0, r1 = int(cu_rows[b]), int(cu_rows[b + 1])
@@ -225,16 +230,19 @@ class CpuKernels:
                 kr = (kr / torch.sqrt((kr * kr).sum(-1, keepdim=True) + unit_eps)).repeat_interleave(rep, 0)
                 vr = v[r].float().reshape(heads, value_dim)
                 bt = torch.sigmoid(beta[r].float())
-                g = torch.exp(-torch.exp(a_log) * torch.nn.functional.softplus(a[r].float() + dt_bias, threshold=1e9))
-                s.mul_(g[:, None, None])
+                step = torch.nn.functional.softplus(a[r].float() + dt_bias, threshold=1e9)
+                if channel_decay:
+                    s.mul_(torch.exp(-torch.exp(a_log)[:, None] * step.reshape(heads, key_dim))[:, None, :])
+                else:
+                    s.mul_(torch.exp(-torch.exp(a_log) * step)[:, None, None])
                 u = bt[:, None] * (vr - (s * kr[:, None, :]).sum(-1))
                 s.add_(u[:, :, None] * kr[:, None, :])
                 out[r] = (s * qr[:, None, :]).sum(-1).reshape(-1)
 
-    def gated_rmsnorm(self, y, z, weight, eps, group, out, gate_first=True):
+    def gated_rmsnorm(self, y, z, weight, eps, group, out, gate_first=True, gate="silu"):
         rows, n = y.shape
         zf = z.float()
-        gate = zf / (1 + torch.exp(-zf))
+        gate = torch.sigmoid(zf) if gate == "sigmoid" else zf / (1 + torch.exp(-zf))
         v = y.float() * gate if gate_first else y.float()
         v = v.reshape(rows, n // group, group)
         v = (v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps)).reshape(rows, n)
@@ -300,6 +308,37 @@ class CpuKernels:
         for h in range(heads):
             out[:, h * out_head_stride : h * out_head_stride + size] = v[:, h].to(out.dtype)
 
+    def rotary_qkv(self, src, q_out, k_out, v_out, heads, kv_heads, key_dim, value_dim, dims, interleaved, freqs,
+                   magnitude, norm_eps, row_pos):
+        rows = src.shape[0]
+        n_rot = (heads + kv_heads) * key_dim
+        turned = torch.empty((rows, n_rot), dtype=torch.float32)
+        if dims:
+            self.rotary(src[:, :n_rot], turned, heads + kv_heads, key_dim, key_dim, dims, interleaved, freqs, magnitude,
+                        row_pos)
+        else:
+            turned.copy_(src[:, :n_rot].float())
+        t = turned.reshape(rows, heads + kv_heads, key_dim)
+        if norm_eps is not None:
+            t = t / torch.sqrt((t * t).mean(-1, keepdim=True) + norm_eps)
+        q_out.copy_(t[:, :heads].reshape(rows, -1).to(q_out.dtype))
+        k_out.copy_(t[:, heads:].reshape(rows, -1).to(k_out.dtype))
+        v_out.copy_(src[:, n_rot:].to(v_out.dtype))
+
+    def postnorm_residual(self, x, y, scales, weight, eps, extra=None, next_weight=None, next_eps=0.0, h=None):
+        pieces = y.float() if y.dim() == 3 else y.float()[None]
+        total = pieces[0] * scales[0]
+        for piece, sc in zip(pieces[1:], scales[1:]):
+            total = total + piece * sc
+        x += total / torch.sqrt((total * total).mean(-1, keepdim=True) + eps) * weight
+        if extra is not None:
+            x += extra
+        if h is not None:
+            h.copy_((x / torch.sqrt((x * x).mean(-1, keepdim=True) + next_eps) * next_weight).to(h.dtype))
+
+    def scale(self, x, factor):
+        x *= factor
+
     def linear_heads(self, x, w, out, heads, out_head_stride):
         n, k = w.shape[1], w.shape[2]
         for h in range(heads):
@@ -319,23 +358,36 @@ class CpuKernels:
                 s.mul_(decay[:, None, :]).add_(vr[:, :, None] * kr[:, None, :])
                 out[r] = (s * qr[:, None, :]).sum(-1).reshape(-1)
 
-    def moe_route(self, logits, route, top, renormalize=False):
+    def moe_route(self, logits, route, top, renormalize=False, correction=None, groups=0, keep=0):
         s = torch.sigmoid(logits.float())
+        c = s + correction if correction is not None else s
+        experts = s.shape[1]
         route.fill_(-1.0)
         for r in range(s.shape[0]):
-            chosen = sorted(range(s.shape[1]), key=lambda e: (-float(s[r, e]), e))[:top]
+            allowed = list(range(experts))
+            if groups > 1 and keep < groups:
+                per = experts // groups
+                marks = [sum(sorted((float(c[r, e]) for e in range(g * per, (g + 1) * per)), reverse=True)[:2])
+                         for g in range(groups)]
+                kept = sorted(range(groups), key=lambda g: (-marks[g], g))[:keep]
+                allowed = [e for e in allowed if e // per in kept]
+            chosen = sorted(allowed, key=lambda e: (-float(c[r, e]), e))[:top]
             total = sum(float(s[r, e]) for e in chosen) if renormalize else 1.0
             for e in chosen:
                 route[r, e] = s[r, e] / total
 
-    def moe_glu(self, gu, route, out, experts, ff, limit, weight_input=True):
+    def moe_glu(self, gu, route, out, experts, ff, limit, weight_input=True, activation="clamped_swish"):
         rows = gu.shape[0]
         v = gu.float().reshape(rows, experts, 2, ff)
-        w = route.float()[:, :, None]
+        w = route.float().reshape(rows, experts)[:, :, None]
         scale = w if weight_input else torch.ones_like(w)
-        g = torch.clamp(v[:, :, 0] * scale, max=limit)
-        u = torch.clamp(v[:, :, 1] * scale, -limit, limit)
-        y = g * torch.sigmoid(1.702 * g) * (u + 1)
+        if activation == "silu":
+            g = v[:, :, 0] * scale
+            y = g * torch.sigmoid(g) * (v[:, :, 1] * scale)
+        else:
+            g = torch.clamp(v[:, :, 0] * scale, max=limit)
+            u = torch.clamp(v[:, :, 1] * scale, -limit, limit)
+            y = g * torch.sigmoid(1.702 * g) * (u + 1)
         if not weight_input:
             y = y * w
         y = torch.where(w >= 0, y, torch.zeros_like(y))
