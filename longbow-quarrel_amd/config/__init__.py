@@ -1,7 +1,8 @@
 """Typed configurations read from a model folder's config.json."""
 from .base import ConfigError, ModelConfig, read_config_json
 from .llama import LlamaConfig, RopeScaling
+from .mifidra import MifidraConfig
 from .vafodra import VafodraConfig
 from .vupelorn import VupelornConfig
 
-__all__ = ["ConfigError", "ModelConfig", "read_config_json", "LlamaConfig", "RopeScaling", "VafodraConfig", "VupelornConfig"]
+__all__ = ["ConfigError", "ModelConfig", "read_config_json", "LlamaConfig", "MifidraConfig", "RopeScaling", "VafodraConfig", "VupelornConfig"]
