@@ -69,8 +69,7 @@ def mifidra_spec(cfg: MifidraConfig) -> ModelSpec:
         ffn = _feed_forward(cfg, layer, i)
         blocks.append(PartSpec("sandwich_norm", {
             "mixer": _mixer(cfg, layer, i), "mixer_norm": norm(f"l{i}.norm1"), "mixer_out_norm": norm(f"l{i}.norm1b"),
-            "feed_forward": ffn, "ffn_norm": None if ffn is None else norm(f"l{i}.norm2"),
-            "ffn_out_norm": None if ffn is None else norm(f"l{i}.norm2b")}))
+            "feed_forward": ffn, "ffn_norm": norm(f"l{i}.norm2"), "ffn_out_norm": norm(f"l{i}.norm2b")}))
     schedule = tuple(Run(i, add_input=again) for i, again in cfg.run_order())
     return ModelSpec(
         vocab_size=cfg.vocab, width=cfg.width, embedding=token_table("embed", cfg.vocab, cfg.width),

@@ -260,7 +260,7 @@ class SandwichNormBlock(Block):
     All four are RMS norms.  One kernel takes a sublayer's result (the sum of its pieces, each with its scale: two
     mixers side by side, routed experts beside a shared one), norms it, adds it to the 32-bit stream and applies the
     norm that the stream meets next: the feed-forward's, or the next block's first.  The feed-forward may be absent
-    (`feed_forward=None`; its two norms then bind no tensors)."""
+    (`feed_forward=None`; its two norms' weights may then be in a file or not, and are not used)."""
 
     takes_next_norm = True
     takes_next_extra = True  # forward(..., next_extra=t): t is added to the stream after the block's last result
@@ -276,6 +276,8 @@ class SandwichNormBlock(Block):
             raise ValueError("a feed-forward needs the norm ahead of it and the norm of its result")
         self.ffn_norm = build_part(NORMS, ffn_norm) if self.ffn is not None else None
         self.ffn_out_norm = build_part(NORMS, ffn_out_norm) if self.ffn is not None else None
+        # the norms of a feed-forward that is not there: a file may hold their weights all the same; they are not used
+        self.idle_norms = [build_part(NORMS, n) for n in (ffn_norm, ffn_out_norm) if self.ffn is None and n is not None]
         for norm in (self.mixer_norm, self.mixer_out_norm, self.ffn_norm, self.ffn_out_norm):
             if norm is not None and not getattr(norm, "deferrable", False):
                 raise ValueError("the norms around the sublayers must be RMS norms")
@@ -293,7 +295,10 @@ class SandwichNormBlock(Block):
                                  self.ffn_out_norm) if p is not None)
 
     def tensor_specs(self) -> List[TensorSpec]:
-        return [s for p in self.parts() for s in p.tensor_specs()]
+        specs = [s for p in self.parts() for s in p.tensor_specs()]
+        for idle in self.idle_norms:
+            specs += [dataclasses.replace(s, optional=True) for s in idle.tensor_specs()]
+        return specs
 
     def bind(self, tensors: Mapping[str, torch.Tensor], env: BuildEnv) -> None:
         super().bind(tensors, env)
