@@ -32,6 +32,9 @@ the default run is not changed by it.
 mixture of experts (per four layers one gated-linear-attention layer, one latent-attention layer with YaRN, one with
 interleaved pairs and one that reads that layer's latent; 8 experts of which a token uses 2, their inner sizes
 such that a token's two experts together are as wide as the Llama shape's feed-forward).
+`--design mifidra`: the same for the design of softmax attention and the gated delta rule side by side (a decay for
+every key channel), with gated units and mixtures of experts in turn; beside the Llama shape and beside the Vafodra
+design of the same sizes, whose gated delta rule (one decay a head) and attention are the closest kernels.
 """
 from __future__ import annotations
 
@@ -130,6 +133,26 @@ def vupelorn_config(width: int, layers: int, vocab: int) -> dict:
             "layers": made, "norm": {"eps": 1e-6}, "vocab": vocab, "width": width}
 
 
+def mifidra_config(width: int, layers: int, vocab: int) -> dict:
+    """Layer sizes of a real model for the design: attention heads of 128 (a fourth as many key/value heads, 64
+    entries rotated under YaRN), delta-rule heads of 128 x 128 (half as many q/k heads, four taps, bottlenecks of 64);
+    gated units of 3.5 times the width in the even layers; in the odd ones 8 experts in 4 groups of which 2 are
+    kept, 2 experts a token, each 1.25 times the width, beside a shared expert as wide as the model (3.5 times
+    together).  No stretch of layers runs twice: depth and weights are those of the shapes beside it."""
+    heads = width // 128
+    rot = {"base": 10000.0, "dims": 64, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}
+    left = {"dim": 128, "vdim": 128, "heads": heads, "kv_heads": max(1, heads // 4), "scale": 128 ** -0.5, "rot": rot}
+    right = {"conv": 4, "dim": 128, "vdim": 128, "heads": heads, "kv_heads": max(1, heads // 2), "decay_rank": 64,
+             "gate_rank": 64}
+    mixer = {"left": left, "right": right, "left_scale": 1.0, "right_scale": 1.0}
+    dense = {"kind": "dense", "ff": width * 7 // 2}
+    moe = {"kind": "moe", "expert": {"ff": width * 5 // 4}, "shared": {"ff": width},
+           "router": {"experts": 8, "top": 2, "groups": {"count": 4, "keep": 2}}}
+    made = [{"type": "parallel", "mixer": mixer, "mlp": moe if i % 2 else dense} for i in range(layers)]
+    return {"architecture": "Mifidra", "layers": made, "logit_scale": 1.0, "norm": {"eps": 1e-5}, "vocab": vocab,
+            "width": width}
+
+
 def design_run(args) -> int:
     import torch
 
@@ -144,9 +167,11 @@ def design_run(args) -> int:
     for width in [int(w) for w in args.design_widths.split(",")]:
         llama = dict(CONFIG_8B, hidden_size=width, intermediate_size=width * 7 // 2, num_hidden_layers=layers,
                      num_attention_heads=width // 128, num_key_value_heads=max(1, width // 512), vocab_size=vocab)
-        design = lq.VafodraConfig.from_dict(vafodra_config(width, layers, vocab)) if args.design == "vafodra" \
-            else lq.VupelornConfig.from_dict(vupelorn_config(width, layers, vocab))
-        for name, config in ((args.design, design), ("llama", lq.LlamaConfig.from_dict(llama))):
+        made = {"vafodra": lambda: lq.VafodraConfig.from_dict(vafodra_config(width, layers, vocab)),
+                "vupelorn": lambda: lq.VupelornConfig.from_dict(vupelorn_config(width, layers, vocab)),
+                "mifidra": lambda: lq.MifidraConfig.from_dict(mifidra_config(width, layers, vocab))}
+        beside = [("vafodra", made["vafodra"]())] if args.design == "mifidra" else []
+        for name, config in [(args.design, made[args.design]())] + beside + [("llama", lq.LlamaConfig.from_dict(llama))]:
             engine = lq.random_engine(config, seed=0, dtype=args.dtype, max_tokens=batch * 4096 + n_prefill + 64,
                                       max_slots=batch + 1, max_sequence_tokens=max(4096, n_prefill))
             prompt = lambda n: torch.randint(0, vocab, (n,), generator=gen).tolist()
@@ -205,7 +230,7 @@ def design_run(args) -> int:
             del engine, backend, timed
             torch.cuda.empty_cache()
     print(json.dumps({"metric": f"prefill and decode tok/s of the {args.design.capitalize()} design beside the Llama shape "
-                                "of equal size",
+                                "of equal size" + (" and the Vafodra design" if args.design == "mifidra" else ""),
                       "dtype": args.dtype, "data": "synthetic: random weights from a seed, uniform random token ids",
                       "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "results": results}), flush=True)
     return 0
@@ -235,7 +260,7 @@ def main() -> int:
                     help="float32: the true 32-bit path (use --layers with the larger shapes)")
     ap.add_argument("--context", type=int, default=0,
                     help="tokens a sequence may hold (default: the shape's 8192); for decoding over longer prompts")
-    ap.add_argument("--design", choices=["vafodra", "vupelorn"], default=None,
+    ap.add_argument("--design", choices=["vafodra", "vupelorn", "mifidra"], default=None,
                     help="measure this design beside the Llama shape of equal size instead of the default workload")
     ap.add_argument("--design-widths", default="2048,4096", help="model widths of --design, with commas between them")
     args = ap.parse_args()

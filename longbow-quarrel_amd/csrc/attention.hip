@@ -58,6 +58,13 @@ extern "C" int lq_attention_folds_rope(int dtype, int nh, int nkv, int hd, int b
   return hd % 64 == 0 && lq_attention_mfma_accepts(dtype, nh, nkv, hd, block_size, 8, 8, nullptr, nullptr, 1);
 }
 
+// Whether launches of this shape, of prompts and of single tokens alike, run on the matrix-core kernel (operands that
+// are dense rows of heads * head_dim, aligned as an allocation is).
+extern "C" int lq_attention_on_matrix_cores(int dtype, int nh, int nkv, int hd, int block_size) {
+  return nh > 0 && nkv > 0 && nh % nkv == 0 && (nh * hd) % 8 == 0 &&
+         lq_attention_mfma_accepts(dtype, nh, nkv, hd, block_size, 8, 8, nullptr, nullptr, 1);
+}
+
 // `decode` != 0 promises one row per sequence; `max_len` is then an upper bound of the
 // sequences' lengths after this step (it sizes the split grid, not the result).  `tickets` are
 // counters that are zero between launches (a launch leaves them so): one for each row and kv head.

@@ -999,6 +999,69 @@ __global__ __launch_bounds__(256) void postnorm_residual_kernel(float* __restric
   for (int i = threadIdx.x; i < width; i += 256) h[base + i] = from_f32<T>(x[base + i] * inv2 * next_w[i]);
 }
 
+// The same for rows of up to 256 * 4 * KEEP entries, a multiple of four, all operands 16-byte aligned: a thread keeps
+// its entries (four neighbours at a time) in registers from the first pass on, so that a row is read once; what a
+// single token's step waits for is the passes' round trips, not the bytes.
+template <typename T, int KEEP>
+__global__ __launch_bounds__(256) void postnorm_residual_kept_kernel(float* __restrict__ x, NormPieces in, int n_in,
+                                                                     const float* __restrict__ w, float eps,
+                                                                     const float* __restrict__ extra,
+                                                                     const float* __restrict__ next_w, float next_eps,
+                                                                     T* __restrict__ h, int width) {
+  __shared__ float red[16];
+  const long long base = (long long)blockIdx.x * width;
+  const int n4 = width >> 2;
+  float4 v[KEEP];
+  float acc = 0.f;
+#pragma unroll
+  for (int j = 0; j < KEEP; ++j) {
+    const int i = threadIdx.x + j * 256;
+    if (i < n4) {
+      float4 a = reinterpret_cast<const float4*>(in.y[0] + base)[i];
+      a.x *= in.scale[0], a.y *= in.scale[0], a.z *= in.scale[0], a.w *= in.scale[0];
+#pragma unroll
+      for (int p = 1; p < 4; ++p)
+        if (p < n_in) {
+          const float4 b = reinterpret_cast<const float4*>(in.y[p] + base)[i];
+          a.x = fmaf(in.scale[p], b.x, a.x), a.y = fmaf(in.scale[p], b.y, a.y);
+          a.z = fmaf(in.scale[p], b.z, a.z), a.w = fmaf(in.scale[p], b.w, a.w);
+        }
+      v[j] = a;
+      acc = fmaf(a.x, a.x, acc), acc = fmaf(a.y, a.y, acc), acc = fmaf(a.z, a.z, acc), acc = fmaf(a.w, a.w, acc);
+    }
+  }
+  const float inv = 1.f / sqrtf(block_sum(acc, red) / (float)width + eps);
+  float acc2 = 0.f;
+#pragma unroll
+  for (int j = 0; j < KEEP; ++j) {
+    const int i = threadIdx.x + j * 256;
+    if (i < n4) {
+      float4 a = reinterpret_cast<const float4*>(x + base)[i];
+      const float4 ww = reinterpret_cast<const float4*>(w)[i];
+      a.x += v[j].x * inv * ww.x, a.y += v[j].y * inv * ww.y, a.z += v[j].z * inv * ww.z, a.w += v[j].w * inv * ww.w;
+      if (extra != nullptr) {
+        const float4 e = reinterpret_cast<const float4*>(extra + base)[i];
+        a.x += e.x, a.y += e.y, a.z += e.z, a.w += e.w;
+      }
+      reinterpret_cast<float4*>(x + base)[i] = a;
+      v[j] = a;
+      acc2 = fmaf(a.x, a.x, acc2), acc2 = fmaf(a.y, a.y, acc2), acc2 = fmaf(a.z, a.z, acc2), acc2 = fmaf(a.w, a.w, acc2);
+    }
+  }
+  if (h == nullptr) return;
+  const float inv2 = 1.f / sqrtf(block_sum(acc2, red) / (float)width + next_eps);
+#pragma unroll
+  for (int j = 0; j < KEEP; ++j) {
+    const int i = threadIdx.x + j * 256;
+    if (i < n4) {
+      const float4 ww = reinterpret_cast<const float4*>(next_w)[i];
+      T* o = h + base + 4 * (long long)i;
+      o[0] = from_f32<T>(v[j].x * inv2 * ww.x), o[1] = from_f32<T>(v[j].y * inv2 * ww.y);
+      o[2] = from_f32<T>(v[j].z * inv2 * ww.z), o[3] = from_f32<T>(v[j].w * inv2 * ww.w);
+    }
+  }
+}
+
 __global__ __launch_bounds__(256) void scale_kernel(float* __restrict__ x, float s, long long n) {
   const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
   if (i < n) x[i] *= s;
@@ -1047,11 +1110,21 @@ extern "C" int lq_postnorm_residual(float* x, const float* y, int pieces, long l
   NormPieces in;
   const float sc[4] = {s0, s1, s2, s3};
   for (int i = 0; i < 4; ++i) in.y[i] = y + (i < pieces ? i : 0) * piece_stride, in.scale[i] = sc[i];
-  if (h == nullptr || h_dtype == LQ_F32)
-    postnorm_residual_kernel<float><<<rows, 256, 0, stream>>>(x, in, pieces, w, eps, extra, next_w, next_eps, (float*)h, width);
-  else if (h_dtype == LQ_BF16)
-    postnorm_residual_kernel<bf16_t><<<rows, 256, 0, stream>>>(x, in, pieces, w, eps, extra, next_w, next_eps, (bf16_t*)h, width);
-  else LQ_REQUIRE(false, "postnorm_residual: unknown dtype %d", h_dtype);
+  bool aligned = width % 4 == 0 && width <= 256 * 4 * 8 && (uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0 &&
+                 (uintptr_t)extra % 16 == 0 && (uintptr_t)next_w % 16 == 0;
+  for (int p = 0; p < pieces; ++p) aligned = aligned && (uintptr_t)in.y[p] % 16 == 0;
+  const bool wide = width > 256 * 4 * 4;
+#define LQ_POSTNORM(KERNEL, T) KERNEL<<<rows, 256, 0, stream>>>(x, in, pieces, w, eps, extra, next_w, next_eps, (T*)h, width)
+  if (h == nullptr || h_dtype == LQ_F32) {
+    if (aligned && wide) LQ_POSTNORM((postnorm_residual_kept_kernel<float, 8>), float);
+    else if (aligned) LQ_POSTNORM((postnorm_residual_kept_kernel<float, 4>), float);
+    else LQ_POSTNORM(postnorm_residual_kernel<float>, float);
+  } else if (h_dtype == LQ_BF16) {
+    if (aligned && wide) LQ_POSTNORM((postnorm_residual_kept_kernel<bf16_t, 8>), bf16_t);
+    else if (aligned) LQ_POSTNORM((postnorm_residual_kept_kernel<bf16_t, 4>), bf16_t);
+    else LQ_POSTNORM(postnorm_residual_kernel<bf16_t>, bf16_t);
+  } else LQ_REQUIRE(false, "postnorm_residual: unknown dtype %d", h_dtype);
+#undef LQ_POSTNORM
   LQ_CHECK_LAUNCH("postnorm_residual");
   return 0;
 }

@@ -65,8 +65,9 @@ __global__ __launch_bounds__(128) void rotary_kernel(const float* __restrict__ s
 // Queries, keys and values of a step's rows, from the 32-bit result of their one product to what the attention
 // kernel and the cache read.  src [rows, (H + G) D + G V]: H query heads, G key heads, G value heads.  Of every query
 // and key head the first `dims` entries are rotated as in `rotary_kernel`; then, with norm_eps >= 0, the whole head
-// is divided by its root mean square over D (eps inside the root); values pass.  One workgroup a row; a wavefront
-// takes a head at a time (its sum of squares is the wavefront's fixed tree, so it depends on the row alone).
+// is divided by its root mean square over D (eps inside the root); values pass.  gridDim.y workgroups a row share
+// its heads and values out (one where the rows alone fill the chip); a wavefront takes a head at a time (its sum of
+// squares is the wavefront's fixed tree, so it depends on the row alone, not on how the heads were shared out).
 template <typename T>
 __global__ __launch_bounds__(256) void rotary_qkv_kernel(const float* __restrict__ src, int lds_, T* __restrict__ q_out,
                                                          int ldq, T* __restrict__ k_out, int ldk, T* __restrict__ v_out,
@@ -89,7 +90,7 @@ __global__ __launch_bounds__(256) void rotary_qkv_kernel(const float* __restrict
   __syncthreads();
   const float* s = src + (long long)r * lds_;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, waves = blockDim.x >> 6;
-  for (int h = wave; h < H + G; h += waves) {
+  for (int h = blockIdx.y * waves + wave; h < H + G; h += waves * gridDim.y) {
     const float* v = s + h * D;
     T* o = h < H ? q_out + (long long)r * ldq + h * D : k_out + (long long)r * ldk + (h - H) * D;
     auto turned = [&](int i) -> float {
@@ -114,7 +115,7 @@ __global__ __launch_bounds__(256) void rotary_qkv_kernel(const float* __restrict
   }
   const float* vs = s + (H + G) * D;
   T* vo = v_out + (long long)r * ldv;
-  for (int e = threadIdx.x; e < G * V; e += blockDim.x) vo[e] = from_f32<T>(vs[e]);
+  for (int e = blockIdx.y * blockDim.x + threadIdx.x; e < G * V; e += blockDim.x * gridDim.y) vo[e] = from_f32<T>(vs[e]);
 }
 
 // A product a head: out[r, h ohs + n] = sum_k x[r, h K + k] w[h, n, k], bfloat16 operands on
@@ -205,12 +206,15 @@ extern "C" int lq_rotary_qkv(const float* src, int lds_, void* q_out, int ldq, v
                  ldv >= kv_heads * value_dim, "rotary_qkv: a row stride is smaller than its row");
   LQ_REQUIRE(src && q_out && k_out && v_out && row_pos && (dims == 0 || freqs), "rotary_qkv: null pointer");
   const size_t lds_bytes = (size_t)dims * sizeof(float);
+  // few rows (single tokens): a wavefront a head, so that no wavefront walks through its heads one after the other
+  const int share = rows >= 512 ? 1 : (lq_ceil_div(heads + kv_heads, 4) < 64 ? lq_ceil_div(heads + kv_heads, 4) : 64);
+  const dim3 grid(rows, share);
   if (out_dtype == LQ_F32)
-    rotary_qkv_kernel<float><<<rows, 256, lds_bytes, stream>>>(src, lds_, (float*)q_out, ldq, (float*)k_out, ldk, (float*)v_out,
+    rotary_qkv_kernel<float><<<grid, 256, lds_bytes, stream>>>(src, lds_, (float*)q_out, ldq, (float*)k_out, ldk, (float*)v_out,
                                                                ldv, heads, kv_heads, key_dim, value_dim, dims, interleaved,
                                                                freqs, magnitude, norm_eps, row_pos);
   else if (out_dtype == LQ_BF16)
-    rotary_qkv_kernel<bf16_t><<<rows, 256, lds_bytes, stream>>>(src, lds_, (bf16_t*)q_out, ldq, (bf16_t*)k_out, ldk,
+    rotary_qkv_kernel<bf16_t><<<grid, 256, lds_bytes, stream>>>(src, lds_, (bf16_t*)q_out, ldq, (bf16_t*)k_out, ldk,
                                                                 (bf16_t*)v_out, ldv, heads, kv_heads, key_dim, value_dim, dims,
                                                                 interleaved, freqs, magnitude, norm_eps, row_pos);
   else LQ_REQUIRE(false, "rotary_qkv: unknown dtype %d", out_dtype);

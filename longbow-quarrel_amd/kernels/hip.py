@@ -20,7 +20,7 @@ from .. import build as _build
 from .dry import query
 
 F32, BF16 = 0, 1
-ABI_VERSION = 8  # lq_abi_version() of the library these wrappers were written for
+ABI_VERSION = 9  # lq_abi_version() of the library these wrappers were written for
 _DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
 
 
@@ -558,6 +558,15 @@ class HipKernels:
             return False
         return bool(self.lib.lq_attention_folds_rope(c_int(_DTYPE_CODE[dtype]), c_int(heads), c_int(kv_heads),
                                                      c_int(head_dim), c_int(block_size)))
+
+    @query
+    def attention_on_matrix_cores(self, dtype: torch.dtype, heads: int, kv_heads: int, head_dim: int, block_size: int) -> bool:
+        """Whether `attention` runs this shape on its matrix-core kernel, prompts and single tokens alike (keys and
+        values of one size, dense rows)."""
+        if self.force_generic or dtype not in _DTYPE_CODE:
+            return False
+        return bool(self.lib.lq_attention_on_matrix_cores(c_int(_DTYPE_CODE[dtype]), c_int(heads), c_int(kv_heads),
+                                                          c_int(head_dim), c_int(block_size)))
 
     @query
     def attention_adds_pieces(self, dtype: torch.dtype, heads: int, kv_heads: int, head_dim: int, block_size: int) -> bool:

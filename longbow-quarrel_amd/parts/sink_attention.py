@@ -115,6 +115,19 @@ class SinkWindowAttention(Mixer):
         # a window that keeps first tokens still gives its middle blocks back
         return KVNeed(self.kv_heads, self.key_dim, self.window, self.value_dim, self.keep_first if self.window else 0)
 
+    def lengths_uneven(self, kernels, lengths) -> bool:
+        ask = getattr(kernels, "decode_lengths_uneven", None)
+        plain = not (self.sink or self.head_gate or self.keep_first or self.window) and self.key_dim == self.value_dim
+        return bool(ask(lengths)) if ask is not None and plain else False
+
+    def _plain_causal(self, kn, ctx: StepContext, cache: LayerCache) -> bool:
+        """Whether this step's attention is the causal kernel's (`attention`): the mask and softmax are plain, and
+        the kernel object runs the shape on its matrix cores (the slower general kernel serves otherwise)."""
+        if self.sink or self.head_gate or self.keep_first or self.key_dim != self.value_dim:
+            return False
+        ask = getattr(kn, "attention_on_matrix_cores", None)
+        return ask is not None and bool(ask(ctx.dtype, self.heads, self.kv_heads, self.key_dim, cache.block_size))
+
     def forward(self, h: torch.Tensor, ctx: StepContext, cache: Optional[LayerCache],
                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
         if cache is None or cache.k is None:
@@ -147,6 +160,18 @@ class SinkWindowAttention(Mixer):
             kn.kv_store(k, v, self.kv_heads, self.key_dim, self.value_dim, ctx.row_pos, ctx.row_seq, ctx.seq_slot,
                         cache.block_table, cache.k, cache.v, cache.block_size)
         att = ctx.ws.alloc((rows, self.o_width), ctx.dtype)
+        if self._plain_causal(kn, ctx, cache):
+            # no sink, gate or kept first tokens, keys and values of one size: the causal kernel on the matrix cores
+            need = kn.attention_workspace(ctx.dtype, rows, self.heads, self.kv_heads, self.key_dim, cache.block_size,
+                                          ctx.decode, ctx.max_len)
+            kn.attention(q, att, self.heads, self.kv_heads, self.key_dim, ctx.row_pos, ctx.row_seq, ctx.seq_slot,
+                         ctx.cu_rows, cache.block_table, cache.k, cache.v, cache.block_size, self.scale, self.window,
+                         decode=ctx.decode, max_len=ctx.max_len,
+                         workspace=ctx.ws.alloc((need,), torch.float32) if need else None, uneven=ctx.uneven)
+            if out is None:
+                out = ctx.ws.alloc((rows, self.width), torch.float32)
+            project(kn, ctx, att, self.w_o, out)
+            return out
         kn.sink_attention(q, att, self.heads, self.kv_heads, self.key_dim, self.value_dim, ctx.row_pos, ctx.row_seq,
                           ctx.seq_slot, cache.block_table, cache.k, cache.v, cache.block_size, self.scale,
                           window=self.window, keep_first=self.keep_first, sink=self.sink, gate=gate,

@@ -86,6 +86,14 @@ CFG_C = _config(1000, 320, 1e-5, 0.25, [
     _layer(_left(8, 8, 32, 64, 0.18, 50000.0), _right(2, 1, 64, 32, 3, 32, 16), 1.0, 0.5, _dense(384)),
     _layer(_left(2, 1, 128, 128, 0.09, 10000.0, 64), _right(8, 8, 16, 16, 2, 8, 8), 0.9, 0.9, _moe(4, 1, 128, None, 64)),
 ])
+# D: attention heads whose keys and values are of one size that the causal matrix-core kernel takes (a bfloat16 run
+# then goes through it, a float32 run through the general kernel)
+CFG_D = _config(500, 256, 1e-5, 0.5, [
+    _layer(_left(8, 2, 64, 64, 0.125, 10000.0, 32, {"factor": 4.0, "original": 128, "fast": 32.0, "slow": 1.0}),
+           _right(2, 1, 32, 32, 4, 16, 16), 0.8, 0.9, _dense(384)),
+    _layer(_left(4, 4, 128, 128, 0.09, 50000.0), _right(2, 2, 16, 64, 3, 8, 16), 1.0, 0.5, _moe(8, 2, 64, (4, 2), 128)),
+    _layer(_left(6, 1, 32, 32, 0.18, 10000.0, 16), _right(4, 2, 32, 16, 2, 8, 8), 0.9, 1.1, None),
+], loop=(0, 2, 2))
 # one mechanism a model: what fails here names its mechanism (the other side of the mixer is weighted with zero)
 CFG_ATTENTION = _config(60, 48, 1e-6, 1.0, [
     _layer(_left(4, 2, 16, 8, 0.3, 200.0, 12, {"factor": 3.0, "original": 20, "fast": 8.0, "slow": 1.0}),
@@ -101,7 +109,7 @@ CFG_LOOP = _config(60, 48, 1e-6, 2.0, [
     _layer(_left(1, 1, 16, 8, 0.2, 100.0), _right(2, 2, 8, 8, 3, 2, 2), 0.7, 0.9, None),
     _layer(_left(2, 2, 8, 16, 0.3, 100.0), _right(2, 1, 8, 8, 2, 3, 3), 0.6, 0.8, _dense(16)),
 ], loop=(0, 2, 3))
-CONFIGS = {"a": CFG_A, "b": CFG_B, "c": CFG_C, "attention": CFG_ATTENTION, "delta": CFG_DELTA, "dense": CFG_DENSE,
+CONFIGS = {"a": CFG_A, "b": CFG_B, "c": CFG_C, "d": CFG_D, "attention": CFG_ATTENTION, "delta": CFG_DELTA, "dense": CFG_DENSE,
            "moe": CFG_MOE, "loop": CFG_LOOP}
 
 

@@ -196,7 +196,7 @@ def test_rotation_of_neighbouring_pairs_and_the_unit_root_mean_square(kn, dtype,
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_norm_of_a_result_in_pieces_added_to_the_stream_with_the_next_norm(kn, dtype):
-    for rows, width in ((9, 200), (1, 50), (70, 256), (3, 4100)):
+    for rows, width in ((9, 200), (1, 50), (70, 256), (3, 4100), (8, 4096), (2, 8200)):
         x = rnd(rows, width, seed=1, std=3.0)
         w, nw = rnd(width, seed=2) + 1, rnd(width, seed=3) + 1
         extra = rnd(rows, width, seed=4)
@@ -409,6 +409,32 @@ def test_bfloat16_decoding_over_long_contexts(cases):
     noise = max(case.noise(t), case.noise(u))
     mc.assert_close_bf16(got, want, noise)
     mc.assert_close_bf16(got, whole.double(), noise)
+
+
+def test_bfloat16_attention_on_the_causal_matrix_core_kernel_and_on_the_general_one(cases, monkeypatch):
+    """Heads whose keys and values are of one size run, in bfloat16, through the causal kernel that the Llama shape
+    uses; the general kernel must give the same up to rounding, in prompts, portions and single tokens over
+    several hundred cached rows, and both must agree with the plain implementation."""
+    from longbow_quarrel_amd.parts.sink_attention import SinkWindowAttention
+    case = cases("d", "bfloat16")
+    calls = []
+    real = case.eng.kernels.attention
+    monkeypatch.setattr(case.eng.kernels, "attention", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+    t = mc.tokens(400, case.vocab, 71)
+    want, noise = case.want(t), case.noise(t)
+    fast = case.run_cut(t, [300, 2, 64])
+    assert len(calls) == 5 * 37  # five layer runs, a prompt, two portions and 34 single tokens
+    mc.assert_close_bf16(fast, want, noise)
+    monkeypatch.setattr(SinkWindowAttention, "_plain_causal", lambda self, kn, ctx, cache: False)
+    general = case.run_cut(t, [300, 2, 64])
+    assert len(calls) == 5 * 37
+    mc.assert_close_bf16(general, want, noise)
+    mc.assert_close_bf16(fast, general.double(), noise)
+    # float32 runs take the general kernel, and sharply
+    case = cases("d")
+    assert mc.err(case.run_cut(t[:200], [150, 2]), case.want(t[:200])) < TOL_F32
+    reqs, wants = mc.greedy(case, n_new=8, prompts=3)
+    assert lq.generate(case.eng, reqs, max_new_tokens=8, use_graphs=True).tokens == wants
 
 
 def test_a_far_key_carries_the_result(cases):
