@@ -735,7 +735,10 @@ constexpr int dch_tokens(int np, int th, int ln) {
   return t >= 16 ? 16 : t >= 8 ? 8 : t >= 4 ? 4 : t >= 2 ? 2 : 1;
 }
 
-template <int LN, int SLAB, int TH>
+// SINGLE: chunks of one token, for a step of single tokens: a workgroup's LDS is then a few hundred bytes where a chunk
+// of 16 tokens takes 50 KB, so all of a compute unit's workgroups are resident at once.  A token's operations and their
+// order are the same either way.
+template <int LN, int SLAB, int TH, bool SINGLE>
 __global__ __launch_bounds__(TH) void delta_channel_scan_kernel(const float* __restrict__ q, int ldq,
                                                                  const float* __restrict__ k, int ldk,
                                                                  const float* __restrict__ v, int ldv,
@@ -747,7 +750,7 @@ __global__ __launch_bounds__(TH) void delta_channel_scan_kernel(const float* __r
                                                                  int ldo, ScanShape sh) {
   extern __shared__ float lds[];
   constexpr int NP = LN * SLAB;  // a shared row in LDS, padded with zeros: entries past N take part as zeros
-  constexpr int TT = dch_tokens(NP, TH, LN);
+  constexpr int TT = SINGLE ? 1 : dch_tokens(NP, TH, LN);
   constexpr int PER = (3 * TT * NP + TH - 1) / TH;
   constexpr int cols = TH / LN;
   constexpr int XPRE = (TT * cols + TH - 1) / TH;
@@ -1129,11 +1132,18 @@ extern "C" int lq_delta_scan(float* q, int ldq, float* k, int ldk, const float* 
   ScanShape sh = {heads, kv_heads, P, Dk, seq_slot, cu_rows};
   if (channel_decay) {
     const int np = cfg.ln * cfg.slab;
-    const size_t lds = 2 * (size_t)dch_tokens(np, cfg.threads, cfg.ln) * (3 * np + 2 * cfg.cols + 1) * sizeof(float);
+    const bool single = rows == batch;  // every sequence brings one token
+    const size_t lds = 2 * (size_t)(single ? 1 : dch_tokens(np, cfg.threads, cfg.ln)) * (3 * np + 2 * cfg.cols + 1) * sizeof(float);
     LQ_REQUIRE(lds <= 64 * 1024, "delta_scan: key size %d is too large", Dk);
-#define LQ_DELTA_CH(LN, SL, TH)                                                                                           \
-  delta_channel_scan_kernel<LN, SL, TH><<<grid, cfg.threads, lds, stream>>>(q, ldq, k, ldk, v, ldv, beta, ldbeta, a, lda, \
-                                                                            dt_bias, a_log, state, out, ldo, sh)
+#define LQ_DELTA_CH(LN, SL, TH)                                                                                          \
+  do {                                                                                                                   \
+    if (single)                                                                                                          \
+      delta_channel_scan_kernel<LN, SL, TH, true><<<grid, cfg.threads, lds, stream>>>(                                   \
+          q, ldq, k, ldk, v, ldv, beta, ldbeta, a, lda, dt_bias, a_log, state, out, ldo, sh);                            \
+    else                                                                                                                 \
+      delta_channel_scan_kernel<LN, SL, TH, false><<<grid, cfg.threads, lds, stream>>>(                                  \
+          q, ldq, k, ldk, v, ldv, beta, ldbeta, a, lda, dt_bias, a_log, state, out, ldo, sh);                            \
+  } while (0)
     LQ_SCAN_LANES(LQ_DELTA_CH)
 #undef LQ_DELTA_CH
     LQ_CHECK_LAUNCH("delta_scan(channel decay)");

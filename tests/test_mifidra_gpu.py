@@ -94,7 +94,7 @@ def test_delta_rule_scan_with_a_decay_for_every_key_channel(kn, sizes):
     state[list(slots)] = 0
     got = [[], []]
     at = [0, 0]
-    for cut in ((1, 7), (2, 1), (30, 1), (1, 10), (11, 0)):
+    for cut in ((1, 7), (1, 1), (2, 1), (30, 1), (1, 9), (10, 0)):  # (one token each: the kernel's form for single tokens)
         live = [i for i in (0, 1) if cut[i]]
         parts = [[t[at[i] : at[i] + cut[i]] for t in seqs[i]] for i in live]
         rows = sum(cut[i] for i in live)
