@@ -83,7 +83,7 @@ CFG_B = _config(97, 50, 1e-5, 1.0, [
 CFG_C = _config(1000, 320, 1e-5, 0.25, [
     _layer(_left(4, 2, 64, 32, 0.12, 10000.0, 32, {"factor": 4.0, "original": 128, "fast": 32.0, "slow": 1.0}),
            _right(4, 2, 32, 64, 4, 16, 32), 0.7, 1.1, _moe(8, 2, 64, (4, 2), 192)),
-    _layer(_left(8, 8, 32, 64, 0.18, 50000.0), _right(2, 1, 64, 32, 3, 32, 16), 1.0, 0.5, _dense(384)),
+    _layer(_left(8, 8, 32, 64, 0.18, 40000.0), _right(2, 1, 64, 32, 3, 32, 16), 1.0, 0.5, _dense(384)),
     _layer(_left(2, 1, 128, 128, 0.09, 10000.0, 64), _right(8, 8, 16, 16, 2, 8, 8), 0.9, 0.9, _moe(4, 1, 128, None, 64)),
 ])
 # D: attention heads whose keys and values are of one size that the causal matrix-core kernel takes (a bfloat16 run
@@ -91,7 +91,7 @@ CFG_C = _config(1000, 320, 1e-5, 0.25, [
 CFG_D = _config(500, 256, 1e-5, 0.5, [
     _layer(_left(8, 2, 64, 64, 0.125, 10000.0, 32, {"factor": 4.0, "original": 128, "fast": 32.0, "slow": 1.0}),
            _right(2, 1, 32, 32, 4, 16, 16), 0.8, 0.9, _dense(384)),
-    _layer(_left(4, 4, 128, 128, 0.09, 50000.0), _right(2, 2, 16, 64, 3, 8, 16), 1.0, 0.5, _moe(8, 2, 64, (4, 2), 128)),
+    _layer(_left(4, 4, 128, 128, 0.09, 40000.0), _right(2, 2, 16, 64, 3, 8, 16), 1.0, 0.5, _moe(8, 2, 64, (4, 2), 128)),
     _layer(_left(6, 1, 32, 32, 0.18, 10000.0, 16), _right(4, 2, 32, 16, 2, 8, 8), 0.9, 1.1, None),
 ], loop=(0, 2, 2))
 # one mechanism a model: what fails here names its mechanism (the other side of the mixer is weighted with zero)
