@@ -16,6 +16,11 @@ pass; `qk_norm_eps` then divides every query and key head by its root mean squar
 are taken in 32-bit on the product's 32-bit result, by one kernel that also leaves q, k and v in the dtype of the
 cache.
 
+`probabilities="bfloat16"` says that a design lets the softmax's weights be rounded to bfloat16 as operands of their
+product with the values (the sums stay 32-bit): plain causal attention with keys and values of one size then runs, in
+a bfloat16 run, on the causal kernel of the matrix cores, several times as fast over a prompt.  The default keeps the
+weights 32-bit through that product.
+
 All projections of h are one matrix product ([q | k | v | gate]).
 """
 from __future__ import annotations
@@ -47,7 +52,8 @@ class SinkWindowAttention(Mixer):
     def __init__(self, width: int, heads: int, kv_heads: int, key_dim: int, value_dim: int, scale: float,
                  prefix: str, window: int = 0, keep_first: int = 0, sink: bool = True, head_gate: bool = False,
                  position: Optional[PartSpec] = None, rotary: Optional[Mapping] = None,
-                 qk_norm_eps: Optional[float] = None, names: Optional[Mapping[str, str]] = None) -> None:
+                 qk_norm_eps: Optional[float] = None, names: Optional[Mapping[str, str]] = None,
+                 probabilities: str = "float32") -> None:
         if heads % kv_heads != 0:
             raise ValueError(f"{heads} heads cannot share {kv_heads} kv heads evenly")
         self.rot_dims, self.rot_interleaved, self.rot_magnitude, self.freq_table = 0, False, 1.0, []
@@ -74,6 +80,9 @@ class SinkWindowAttention(Mixer):
         self.key_dim, self.value_dim = int(key_dim), int(value_dim)
         self.scale, self.window, self.keep_first = float(scale), int(window), int(keep_first)
         self.sink, self.head_gate = bool(sink), bool(head_gate)
+        if probabilities not in ("float32", "bfloat16"):
+            raise ValueError(f"probabilities are 'float32' or 'bfloat16', found {probabilities!r}")
+        self.probabilities = probabilities
         n = {"q": "q", "k": "k", "v": "v", "gate": "g", "o": "o"}
         n.update(names or {})
         self.names: Dict[str, str] = {key: f"{prefix}.{val}" for key, val in n.items()}
@@ -117,13 +126,16 @@ class SinkWindowAttention(Mixer):
 
     def lengths_uneven(self, kernels, lengths) -> bool:
         ask = getattr(kernels, "decode_lengths_uneven", None)
-        plain = not (self.sink or self.head_gate or self.keep_first or self.window) and self.key_dim == self.value_dim
+        plain = not (self.sink or self.head_gate or self.keep_first or self.window) and self.key_dim == self.value_dim \
+            and self.probabilities == "bfloat16"
         return bool(ask(lengths)) if ask is not None and plain else False
 
     def _plain_causal(self, kn, ctx: StepContext, cache: LayerCache) -> bool:
-        """Whether this step's attention is the causal kernel's (`attention`): the mask and softmax are plain, and
-        the kernel object runs the shape on its matrix cores (the slower general kernel serves otherwise)."""
-        if self.sink or self.head_gate or self.keep_first or self.key_dim != self.value_dim:
+        """Whether this step's attention is the causal kernel's (`attention`): the design lets the probabilities be
+        rounded to bfloat16 for their product with the values (that kernel's way; the general kernel keeps them
+        32-bit), the mask and softmax are plain, and the kernel object runs the shape on its matrix cores."""
+        if self.probabilities != "bfloat16" or self.sink or self.head_gate or self.keep_first \
+                or self.key_dim != self.value_dim:
             return False
         ask = getattr(kn, "attention_on_matrix_cores", None)
         return ask is not None and bool(ask(ctx.dtype, self.heads, self.kv_heads, self.key_dim, cache.block_size))

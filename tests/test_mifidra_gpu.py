@@ -411,30 +411,40 @@ def test_bfloat16_decoding_over_long_contexts(cases):
     mc.assert_close_bf16(got, whole.double(), noise)
 
 
-def test_bfloat16_attention_on_the_causal_matrix_core_kernel_and_on_the_general_one(cases, monkeypatch):
-    """Heads whose keys and values are of one size run, in bfloat16, through the causal kernel that the Llama shape
-    uses; the general kernel must give the same up to rounding, in prompts, portions and single tokens over
-    several hundred cached rows, and both must agree with the plain implementation."""
+def test_bfloat16_probabilities_on_the_causal_matrix_core_kernel(tmp_path_factory, monkeypatch):
+    """The design keeps the softmax's weights 32-bit, so its attention runs on the general kernel.  A design that
+    lets them be rounded to bfloat16 for their product with the values (the attention part's `probabilities`) runs
+    heads whose keys and values are of one size, in bfloat16, through the causal kernel that the Llama shape uses:
+    the same up to that rounding, in prompts, portions and single tokens over several hundred cached rows."""
     from longbow_quarrel_amd.parts.sink_attention import SinkWindowAttention
-    case = cases("d", "bfloat16")
+    case = mc.Case(tmp_path_factory.mktemp("mifidra_d"), "d", load, dtype="bfloat16", rounding=True)
     calls = []
     real = case.eng.kernels.attention
     monkeypatch.setattr(case.eng.kernels, "attention", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
     t = mc.tokens(400, case.vocab, 71)
     want, noise = case.want(t), case.noise(t)
+    general = case.run_cut(t, [300, 2, 64])
+    assert not calls
+    mc.assert_close_bf16(general, want, noise)
+    parts = [s for m in case.eng.model._mixers() for s in m.sides if isinstance(s, SinkWindowAttention)]
+    assert len(parts) == 3 and all(p.probabilities == "float32" for p in parts)
+    for p in parts:
+        p.probabilities = "bfloat16"
     fast = case.run_cut(t, [300, 2, 64])
     assert len(calls) == 5 * 37  # five layer runs, a prompt, two portions and 34 single tokens
     mc.assert_close_bf16(fast, want, noise)
-    monkeypatch.setattr(SinkWindowAttention, "_plain_causal", lambda self, kn, ctx, cache: False)
-    general = case.run_cut(t, [300, 2, 64])
-    assert len(calls) == 5 * 37
-    mc.assert_close_bf16(general, want, noise)
     mc.assert_close_bf16(fast, general.double(), noise)
-    # float32 runs take the general kernel, and sharply
-    case = cases("d")
-    assert mc.err(case.run_cut(t[:200], [150, 2]), case.want(t[:200])) < TOL_F32
-    reqs, wants = mc.greedy(case, n_new=8, prompts=3)
-    assert lq.generate(case.eng, reqs, max_new_tokens=8, use_graphs=True).tokens == wants
+    reqs = [mc.tokens(n, case.vocab, 40 + n) for n in (3, 70, 9)]
+    a = lq.generate(case.eng, reqs, max_new_tokens=20, stop_ids=[], use_graphs=False)
+    b = lq.generate(case.eng, reqs, max_new_tokens=20, stop_ids=[], use_graphs=True)
+    assert a.tokens == b.tokens
+    # a float32 run takes the general kernel whatever the part allows
+    case = mc.Case(tmp_path_factory.mktemp("mifidra_d32"), "d", load)
+    for m in case.eng.model._mixers():
+        m.sides[0].probabilities = "bfloat16"
+    calls.clear()
+    monkeypatch.setattr(case.eng.kernels, "attention", lambda *a, **k: calls.append(1))
+    assert mc.err(case.run_cut(t[:200], [150, 2]), case.want(t[:200])) < TOL_F32 and not calls
 
 
 def test_a_far_key_carries_the_result(cases):
