@@ -1,2 +1,2 @@
 """Architectures.  Importing the package registers them."""
-from . import llama, mifidra, vafodra, vupelorn  # noqa: F401
+from . import llama, mifidra, sofinex, vafodra, vupelorn  # noqa: F401

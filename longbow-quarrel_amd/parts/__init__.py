@@ -3,7 +3,7 @@ from .base import (BLOCKS, EMBEDDINGS, FEED_FORWARDS, LOGIT_STEPS, MATRIX, MIXER
                    VECTOR32, Block, BuildEnv, CacheNeed, Embedding, FeedForward, KVNeed, LayerCache, LogitsStep, Mixer,
                    MultiCache, MultiNeed, Norm, Part, PartSpec, PositionEncoding, Registry, StateNeed, StepContext, TensorSpec, Workspace,
                    build_part, project)
-from . import attention, block, embedding, feedforward, latent_attention, logits, norms, recurrent, rope, sink_attention  # noqa: F401  (registration)
+from . import attention, block, differential_attention, embedding, feedforward, latent_attention, logits, norms, recurrent, rope, sink_attention  # noqa: F401  (registration)
 
 __all__ = [
     "BLOCKS", "EMBEDDINGS", "FEED_FORWARDS", "LOGIT_STEPS", "MATRIX", "MIXERS", "NORMS", "POSITION_ENCODINGS", "TABLE",

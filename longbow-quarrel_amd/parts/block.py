@@ -16,21 +16,29 @@ from .base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Block, BuildEnv, LayerC
 
 @BLOCKS.register("prenorm")
 class PreNormBlock(Block):
-    def __init__(self, mixer: PartSpec, feed_forward: PartSpec, mixer_norm: PartSpec, ffn_norm: PartSpec) -> None:
+    def __init__(self, mixer: PartSpec, feed_forward: Optional[PartSpec], mixer_norm: PartSpec,
+                 ffn_norm: Optional[PartSpec]) -> None:
+        """`feed_forward=None`: the layer is its mixer alone.  The norm of a feed-forward that is absent may be named
+        all the same: its weight may then be in a file or not, and is not used."""
         self.mixer = build_part(MIXERS, mixer)
-        self.ffn = build_part(FEED_FORWARDS, feed_forward)
+        self.ffn = build_part(FEED_FORWARDS, feed_forward) if feed_forward is not None else None
         self.mixer_norm = build_part(NORMS, mixer_norm)
-        self.ffn_norm = build_part(NORMS, ffn_norm)
+        self.ffn_norm = build_part(NORMS, ffn_norm) if ffn_norm is not None else None
+        if self.ffn is not None and self.ffn_norm is None:
+            raise ValueError("a feed-forward needs the norm ahead of it")
 
     @property
     def graph_safe(self) -> bool:
         return all(p.graph_safe for p in self.parts())
 
     def parts(self):
-        return (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn)
+        return tuple(p for p in (self.mixer_norm, self.mixer) + ((self.ffn_norm, self.ffn) if self.ffn is not None else ()))
 
     def tensor_specs(self) -> List[TensorSpec]:
-        return [s for p in self.parts() for s in p.tensor_specs()]
+        specs = [s for p in self.parts() for s in p.tensor_specs()]
+        if self.ffn is None and self.ffn_norm is not None:
+            specs += [dataclasses.replace(s, optional=True) for s in self.ffn_norm.tensor_specs()]
+        return specs
 
     def bind(self, tensors: Mapping[str, torch.Tensor], env: BuildEnv) -> None:
         super().bind(tensors, env)
@@ -57,11 +65,13 @@ class PreNormBlock(Block):
     def forward(self, x: torch.Tensor, pending, ctx: StepContext, cache: Optional[LayerCache], next_norm=None):
         h = self._normed(self.mixer_norm, x, pending, ctx, self.mixer)
         if self.mixer.takes_residual_sink:
-            sink = ResidualSink(x, self.ffn_norm)
+            sink = ResidualSink(x, self.ffn_norm if self.ffn is not None else next_norm)
             pending = self.mixer.forward(h, ctx, cache, sink=sink)
             pending = sink.stats if pending is None else pending
         else:
             pending = self.mixer.forward(h, ctx, cache)
+        if self.ffn is None:
+            return pending
         h = self._normed(self.ffn_norm, x, pending, ctx, self.ffn)
         if self.ffn.takes_residual_sink:
             sink = ResidualSink(x, next_norm)

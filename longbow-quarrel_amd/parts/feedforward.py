@@ -136,6 +136,46 @@ class GatedLinearUnit(FeedForward):
         return out
 
 
+@FEED_FORWARDS.register("mlp")
+class PlainFeedForward(FeedForward):
+    """down(act(up(h))): two matrices, no gate and no biases; `activation` "gelu" (the exact one, with the error
+    function), "gelu_tanh", "silu" or "relu".  The activation reads the first product's 32-bit result."""
+
+    graph_safe = True
+    takes_out = True
+    ACTIVATIONS = ("gelu", "gelu_tanh", "silu", "relu")
+
+    def __init__(self, width: int, inner: int, prefix: str, activation: str = "gelu",
+                 names: Optional[Mapping[str, str]] = None) -> None:
+        if activation not in self.ACTIVATIONS:
+            raise ValueError(f"unknown activation {activation!r}; known: {', '.join(self.ACTIVATIONS)}")
+        self.width, self.inner, self.activation = int(width), int(inner), activation
+        n = {"up": "up", "down": "down"}
+        n.update(names or {})
+        self.names: Dict[str, str] = {key: f"{prefix}.{val}" for key, val in n.items()}
+        self.w_up = self.w_down = None
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [TensorSpec(self.names["up"], (self.inner, self.width)),
+                TensorSpec(self.names["down"], (self.width, self.inner))]
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], env: BuildEnv) -> None:
+        super().bind(tensors, env)
+        self.w_up = product_weight(env, tensors[self.names["up"]])
+        self.w_down = product_weight(env, tensors[self.names["down"]])
+
+    def forward(self, h, ctx: StepContext, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        kn, rows = ctx.kernels, h.shape[0]
+        u = ctx.ws.alloc((rows, (self.inner + 3) // 4 * 4), torch.float32)[:, : self.inner]
+        project(kn, ctx, h, self.w_up, u)
+        act = ctx.ws.alloc((rows, self.inner), ctx.dtype)
+        kn.activation(u, act, self.activation)
+        if out is None:
+            out = ctx.ws.alloc((rows, self.width), torch.float32)
+        project(kn, ctx, act, self.w_down, out)
+        return out
+
+
 @FEED_FORWARDS.register("moe")
 class MixtureOfExperts(FeedForward):
     """`experts` small gated feed-forwards of which every token uses `top`, chosen by a router.
@@ -153,7 +193,15 @@ class MixtureOfExperts(FeedForward):
     alone; the weights stay the scores.  `groups` / `keep`: the experts form `groups` equal groups of neighbours, a
     group's mark is the sum of its two largest choice scores, and only experts of the `keep` best groups can be
     chosen.  `shared_inner`: one more expert of that inner size (`<prefix>.shared.*`, the same form) runs for every
-    token with weight one, and is added.
+    token with weight one, and is added.  `shared_gate`: the shared expert's result is multiplied by the sigmoid of
+    one more projection of the input, a number a token (`<prefix>.shared.sg`, [1, width]).
+
+    `scoring` "softmax": s = softmax(z) over all the router's outputs in the place of the sigmoid.  `group_mark`
+    "max": a group's mark is its largest choice score (the default, "top2", is the sum of its two largest); experts
+    outside the kept groups cannot be chosen whatever their choice scores (which may be negative).  `renormalize_eps`
+    is added to the chosen scores' sum before the division.  `identity`: so many more outputs of the router, behind
+    the experts', stand for experts without tensors that hand their input on (times the weight); they take part in
+    the scores, the groups and the choice like the others.
 
     How it runs.  The experts' gate and up matrices are one matrix [experts * 2 ff, width] and their down matrices
     one [width, experts * ff]: with the activations of the experts that a token did not choose set to zero, the down
@@ -174,8 +222,18 @@ class MixtureOfExperts(FeedForward):
     def __init__(self, width: int, experts: int, top: int, inner: int, prefix: str, limit: float = 0.0,
                  weight_input: bool = True, renormalize: bool = False, activation: str = "clamped_swish",
                  correction: bool = False, groups: int = 0, keep: int = 0, shared_inner: int = 0,
-                 names: Optional[Mapping[str, str]] = None) -> None:
+                 names: Optional[Mapping[str, str]] = None, scoring: str = "sigmoid", group_mark: str = "top2",
+                 renormalize_eps: float = 0.0, identity: int = 0, shared_gate: bool = False) -> None:
         self.width, self.experts, self.top, self.inner = int(width), int(experts), int(top), int(inner)
+        self.scoring, self.group_mark, self.renormalize_eps = scoring, group_mark, float(renormalize_eps)
+        self.identity, self.shared_gate = int(identity), bool(shared_gate)
+        self.outputs = self.experts + self.identity  # what the router scores
+        if scoring not in ("sigmoid", "softmax") or group_mark not in ("top2", "max"):
+            raise ValueError(f"scoring is 'sigmoid' or 'softmax' ({scoring!r}), a group's mark 'top2' or 'max' ({group_mark!r})")
+        if self.identity < 0 or (self.identity and weight_input):
+            raise ValueError("identity experts: none or more, and the weight on the experts' results")
+        if self.shared_gate and not shared_inner:
+            raise ValueError("a gate on the shared expert needs a shared expert")
         self.limit, self.weight_input, self.renormalize = float(limit), bool(weight_input), bool(renormalize)
         self.activation, self.correction = activation, bool(correction)
         self.groups, self.keep, self.shared_inner = int(groups), int(keep), int(shared_inner)
@@ -183,17 +241,17 @@ class MixtureOfExperts(FeedForward):
             raise ValueError(f"unknown activation {activation!r}; known: {', '.join(self.ACTIVATIONS)}")
         if self.shared_inner and activation != "silu":
             raise ValueError("a shared expert is built for the 'silu' activation only")
-        if not 1 <= self.top <= self.experts:
-            raise ValueError(f"{top} of {experts} experts cannot be chosen")
+        if not 1 <= self.top <= self.outputs:
+            raise ValueError(f"{top} of {self.outputs} experts cannot be chosen")
         if self.groups > 1:
-            if self.experts % self.groups or not 1 <= self.keep <= self.groups or self.groups > 64:
-                raise ValueError(f"{experts} experts do not form {groups} equal groups of which {keep} are kept")
-            if self.keep * (self.experts // self.groups) < self.top:
-                raise ValueError(f"{keep} groups of {self.experts // self.groups} experts cannot give {top} experts")
+            if self.outputs % self.groups or not 1 <= self.keep <= self.groups or self.groups > 64:
+                raise ValueError(f"{self.outputs} experts do not form {groups} equal groups of which {keep} are kept")
+            if self.keep * (self.outputs // self.groups) < self.top:
+                raise ValueError(f"{keep} groups of {self.outputs // self.groups} experts cannot give {top} experts")
         else:
             self.groups = self.keep = 0
         n = {"router": "router", "expert": "e{}", "gate": "gate", "up": "up", "down": "down",
-             "correction": "correction", "shared": "shared"}
+             "correction": "correction", "shared": "shared", "shared_gate": "sg"}
         n.update(names or {})
         self.prefix, self.n = prefix, n
         self.w_correction: Optional[torch.Tensor] = None
@@ -210,13 +268,15 @@ class MixtureOfExperts(FeedForward):
             specs += [TensorSpec(self._name(e, "gate"), (self.inner, self.width)),
                       TensorSpec(self._name(e, "up"), (self.inner, self.width)),
                       TensorSpec(self._name(e, "down"), (self.width, self.inner))]
-        specs.append(TensorSpec(f"{self.prefix}.{self.n['router']}", (self.experts, self.width)))
+        specs.append(TensorSpec(f"{self.prefix}.{self.n['router']}", (self.outputs, self.width)))
         if self.correction:
-            specs.append(TensorSpec(f"{self.prefix}.{self.n['correction']}", (self.experts,), kind=VECTOR32))
+            specs.append(TensorSpec(f"{self.prefix}.{self.n['correction']}", (self.outputs,), kind=VECTOR32))
         if self.shared_inner:
             specs += [TensorSpec(self._shared_name("gate"), (self.shared_inner, self.width)),
                       TensorSpec(self._shared_name("up"), (self.shared_inner, self.width)),
                       TensorSpec(self._shared_name("down"), (self.width, self.shared_inner))]
+        if self.shared_gate:
+            specs.append(TensorSpec(self._shared_name("shared_gate"), (1, self.width)))
         return specs
 
     def bind(self, tensors: Mapping[str, torch.Tensor], env: BuildEnv) -> None:
@@ -252,11 +312,20 @@ class MixtureOfExperts(FeedForward):
             self.w_correction = tensors[f"{self.prefix}.{self.n['correction']}"].contiguous()
         # the router's product as it is stored: bfloat16 operands multiply exactly into 32-bit sums, and its result
         # (the logits) and everything after it are 32-bit
-        self.w_router = tensors[f"{self.prefix}.{self.n['router']}"].contiguous()
+        self.w_router = tensors[f"{self.prefix}.{self.n['router']}"]
+        if self.shared_gate:  # the gate's logit rides in the router's product, as one more row behind its own
+            sg = tensors[self._shared_name("shared_gate")]
+            if sg.dtype != self.w_router.dtype:
+                raise ValueError(f"{self._shared_name('shared_gate')}: stored in another dtype than the router")
+            self.w_router = torch.cat([self.w_router, sg.reshape(1, self.width)], dim=0)
+        self.w_router = self.w_router.contiguous()
 
     def _route(self, h, ctx: StepContext) -> torch.Tensor:
-        kn, rows, E = ctx.kernels, h.shape[0], self.experts
-        z = ctx.ws.alloc((rows, (E + 3) // 4 * 4), torch.float32)[:, :E]
+        """The weight of every expert for every row (-1: not chosen).  Leaves the identity experts' weights and the
+        shared expert's gate logits of this step in `self._step`."""
+        kn, rows, E, N = ctx.kernels, h.shape[0], self.experts, self.outputs
+        nz = N + (1 if self.shared_gate else 0)
+        z = ctx.ws.alloc((rows, (nz + 3) // 4 * 4), torch.float32)[:, :nz]
         project(kn, ctx, h, self.w_router, z)
         route = ctx.ws.alloc((rows, E), torch.float32)  # the weight of a chosen expert, -1 for the others
         more = {}
@@ -264,16 +333,36 @@ class MixtureOfExperts(FeedForward):
             more["correction"] = self.w_correction
         if self.groups > 1:
             more.update(groups=self.groups, keep=self.keep)
-        kn.moe_route(z, route, self.top, self.renormalize, **more)
+        if self.scoring != "sigmoid":
+            more["scoring"] = self.scoring
+        if self.group_mark != "top2":
+            more["group_mark"] = self.group_mark
+        if self.renormalize_eps:
+            more["renormalize_eps"] = self.renormalize_eps
+        passed = None
+        if self.identity:
+            passed = more["identity"] = ctx.ws.alloc((rows, self.identity), torch.float32)
+        kn.moe_route(z[:, :N], route, self.top, self.renormalize, **more)
+        self._step = (passed, z[:, N:] if self.shared_gate else None)
         return route
 
+    def _pass_on(self, h, out, ctx: StepContext) -> None:
+        """The identity experts' share: out += h * (the sum of the chosen identity experts' weights)."""
+        passed = self._step[0]
+        if passed is not None:
+            ctx.kernels.moe_identity(h, passed, out)
+
     def _sorts(self, rows: int, ctx: StepContext) -> bool:
-        return rows >= self.sort_from_rows and not ctx.decode and not ctx.dry and self.experts > self.top \
+        return rows >= self.sort_from_rows and not ctx.decode and not ctx.dry and self.outputs > self.top \
             and getattr(ctx.kernels, "moe_sort", None) is not None
 
     def _unit(self, gu, act, ctx: StepContext) -> None:
-        """The shared expert's activation (weight one, no routing)."""
-        ctx.kernels.glu(gu, act, "silu")
+        """The shared expert's activation (no routing; weight one, or the sigmoid of its gate's logit)."""
+        gate = self._step[1]
+        if gate is not None:
+            ctx.kernels.glu(gu, act, "silu", row_gate=gate)
+        else:
+            ctx.kernels.glu(gu, act, "silu")
 
     def forward_pieces(self, h, ctx: StepContext):
         """The result in pieces [n, rows, width] that the caller adds: the routed experts' sum, and the shared
@@ -285,6 +374,7 @@ class MixtureOfExperts(FeedForward):
             return out, (1.0,)
         out = ctx.ws.alloc((2, rows, self.width), torch.float32)
         self._sorted(h, self._route(h, ctx), out[0], ctx)
+        self._pass_on(h, out[0], ctx)
         self._shared(h, out[1], ctx)
         return out, (1.0, 1.0)
 
@@ -304,6 +394,7 @@ class MixtureOfExperts(FeedForward):
             out = ctx.ws.alloc((rows, self.width), torch.float32)
         if self._sorts(rows, ctx):
             self._sorted(h, route, out, ctx)
+            self._pass_on(h, out, ctx)
             if ffs:
                 extra = ctx.ws.alloc((rows, self.width), torch.float32)
                 self._shared(h, extra, ctx)
@@ -319,6 +410,7 @@ class MixtureOfExperts(FeedForward):
         if ffs:
             self._unit(gu[:, E * 2 * ff :], act[:, E * ff :], ctx)
         project(kn, ctx, act, self.w_down, out)
+        self._pass_on(h, out, ctx)
         return out
 
     def _sorted(self, h, route, out, ctx: StepContext) -> None:

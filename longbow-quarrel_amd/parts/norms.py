@@ -1,7 +1,9 @@
 """RMSNorm: y = x / sqrt(mean(x^2) + eps) * w, eps inside the root, the weight
 after the normalisation (internal/device/kernels.metal:905-942; host twin
 internal/device/cpu_ref.go:63-83).  Statistics in 32-bit, weight held in 32-bit
-(internal/engine/engine.go:788-792 promotes norm weights the same way)."""
+(internal/engine/engine.go:788-792 promotes norm weights the same way).
+`offset`: the stored weight lies around zero and the norm multiplies by offset + w (a design that stores its gains
+as 1 + w names offset = 1); the sum is made once, in 32-bit, when the weights are bound."""
 from __future__ import annotations
 
 from typing import List, Mapping, Optional
@@ -16,18 +18,20 @@ class RMSNorm(Norm):
     graph_safe = True
     deferrable = True  # a consumer may apply it itself from x, weight, eps and the rows' sums of squares
 
-    def __init__(self, width: int, eps: float, name: str) -> None:
+    def __init__(self, width: int, eps: float, name: str, offset: float = 0.0) -> None:
         self.width = int(width)
         self.eps = float(eps)
         self.name = name
+        self.offset = float(offset)
         self.weight: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> List[TensorSpec]:
-        return [TensorSpec(self.name, (self.width,), kind=VECTOR32, init="around_one")]
+        return [TensorSpec(self.name, (self.width,), kind=VECTOR32, init="normal" if self.offset else "around_one")]
 
     def bind(self, tensors: Mapping[str, torch.Tensor], env: BuildEnv) -> None:
         super().bind(tensors, env)
-        self.weight = tensors[self.name].contiguous()
+        w = tensors[self.name]
+        self.weight = (w + self.offset if self.offset else w).contiguous()
 
     def forward(self, x: torch.Tensor, ctx: StepContext, delta: Optional[torch.Tensor] = None) -> torch.Tensor:
         out = ctx.ws.alloc(x.shape, ctx.dtype)

@@ -5,7 +5,8 @@ differ); query head h reads kv head h // (heads / kv_heads).  Position i sees po
 (i - j < window or j < keep_first); window = 0 means every earlier position.  With `sink` the softmax has one
 more term in its denominator, a key of score 0 that carries no value: p_j = e^(s_j) / (1 + sum e^(s_j)), so a
 query may look at nothing (Xiao, Tian, Chen, Han, Lewis: "Efficient Streaming Language Models with Attention
-Sinks" keeps first tokens for the same purpose).  With `head_gate` every head's result is multiplied by the
+Sinks" keeps first tokens for the same purpose).  `sink="learned"`: the term is e^(b_h) with a stored number b_h for
+every query head (`<prefix>.sink`), which is not scaled: p_j = e^(s_j) / (e^(b_h) + sum e^(s_j)).  With `head_gate` every head's result is multiplied by the
 sigmoid of one more projection of h, a number per head.  Scores, probabilities and the sums over values are
 32-bit whatever the run's dtype.  A position encoding is optional (`position=None`: positions do not enter
 the scores).
@@ -29,7 +30,7 @@ from typing import Dict, List, Mapping, Optional
 
 import torch
 
-from .base import (MIXERS, POSITION_ENCODINGS, BuildEnv, KVNeed, LayerCache, Mixer, PartSpec, StepContext,
+from .base import (MIXERS, POSITION_ENCODINGS, VECTOR32, BuildEnv, KVNeed, LayerCache, Mixer, PartSpec, StepContext,
                    TensorSpec, build_part, product_weight, project)
 from .rope import rotary_frequencies, rotary_magnitude
 
@@ -50,7 +51,7 @@ class SinkWindowAttention(Mixer):
     takes_out = True
 
     def __init__(self, width: int, heads: int, kv_heads: int, key_dim: int, value_dim: int, scale: float,
-                 prefix: str, window: int = 0, keep_first: int = 0, sink: bool = True, head_gate: bool = False,
+                 prefix: str, window: int = 0, keep_first: int = 0, sink=True, head_gate: bool = False,
                  position: Optional[PartSpec] = None, rotary: Optional[Mapping] = None,
                  qk_norm_eps: Optional[float] = None, names: Optional[Mapping[str, str]] = None,
                  probabilities: str = "float32") -> None:
@@ -79,11 +80,14 @@ class SinkWindowAttention(Mixer):
         self.width, self.heads, self.kv_heads = int(width), int(heads), int(kv_heads)
         self.key_dim, self.value_dim = int(key_dim), int(value_dim)
         self.scale, self.window, self.keep_first = float(scale), int(window), int(keep_first)
-        self.sink, self.head_gate = bool(sink), bool(head_gate)
+        if sink not in (True, False, "learned"):
+            raise ValueError(f"the sink is True (a score of 0), False or 'learned' (a stored score a head), found {sink!r}")
+        self.sink, self.head_gate, self.learned_sink = bool(sink), bool(head_gate), sink == "learned"
+        self.sink_w: Optional[torch.Tensor] = None
         if probabilities not in ("float32", "bfloat16"):
             raise ValueError(f"probabilities are 'float32' or 'bfloat16', found {probabilities!r}")
         self.probabilities = probabilities
-        n = {"q": "q", "k": "k", "v": "v", "gate": "g", "o": "o"}
+        n = {"q": "q", "k": "k", "v": "v", "gate": "g", "o": "o", "sink": "sink"}
         n.update(names or {})
         self.names: Dict[str, str] = {key: f"{prefix}.{val}" for key, val in n.items()}
         self.position = build_part(POSITION_ENCODINGS, position) if position is not None else None
@@ -106,6 +110,8 @@ class SinkWindowAttention(Mixer):
         ]
         if self.head_gate:
             specs.append(TensorSpec(self.names["gate"], (self.heads, self.width)))
+        if self.learned_sink:
+            specs.append(TensorSpec(self.names["sink"], (self.heads,), kind=VECTOR32))
         specs.append(TensorSpec(self.names["o"], (self.width, self.o_width)))
         return specs + (self.position.tensor_specs() if self.position is not None else [])
 
@@ -116,6 +122,8 @@ class SinkWindowAttention(Mixer):
             raise ValueError(f"{self.names['q']}: the projections of one input are stored in different dtypes")
         self.w_in = product_weight(env, torch.cat(mats, dim=0))
         self.w_o = product_weight(env, tensors[self.names["o"]])
+        if self.learned_sink:
+            self.sink_w = tensors[self.names["sink"]].contiguous()
         if self.position is not None:
             self.position.bind(tensors, env)
         self.freqs = torch.tensor(self.freq_table, dtype=torch.float64, device=env.device) if self.rot_dims else None
@@ -187,7 +195,8 @@ class SinkWindowAttention(Mixer):
         kn.sink_attention(q, att, self.heads, self.kv_heads, self.key_dim, self.value_dim, ctx.row_pos, ctx.row_seq,
                           ctx.seq_slot, cache.block_table, cache.k, cache.v, cache.block_size, self.scale,
                           window=self.window, keep_first=self.keep_first, sink=self.sink, gate=gate,
-                          decode=ctx.decode, **split_scratch(ctx, q.dtype, self.heads, self.kv_heads, self.key_dim,
+                          decode=ctx.decode, **({"sink_values": self.sink_w} if self.learned_sink else {}),
+                          **split_scratch(ctx, q.dtype, self.heads, self.kv_heads, self.key_dim,
                                                              self.value_dim, cache.block_size, self.window,
                                                              self.keep_first))
         if out is None:

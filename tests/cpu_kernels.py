@@ -139,19 +139,31 @@ class CpuKernels:
     def add_scaled(self, x, delta, scale):
         x += self._whole(delta, x) * scale
 
-    def glu(self, gate_up, out, activation, bias=None, tail=0):
+    @staticmethod
+    def _act(g, activation):
+        if activation == "relu":
+            return torch.clamp(g, min=0)
+        if activation == "silu":
+            return g / (1 + torch.exp(-g))
+        if activation == "gelu_tanh":
+            return 0.5 * g * (1 + torch.tanh(math.sqrt(2 / math.pi) * (g + 0.044715 * g * g * g)))
+        if activation == "gelu":
+            return 0.5 * g * (1 + torch.erf(g * math.sqrt(0.5)))
+        raise ValueError(activation)
+
+    def activation(self, x, out, activation):
+        out.copy_(self._act(x.float(), activation).to(out.dtype))
+
+    def glu(self, gate_up, out, activation, bias=None, tail=0, row_gate=None):
         inner = out.shape[1] - tail
         g, u = gate_up[:, :inner].float(), gate_up[:, inner:].float()
         if bias is not None:
             g, u = g + bias[:inner], u + bias[inner:]
-        if activation == "relu":
-            a = torch.clamp(g, min=0)
-        elif activation == "silu":
-            a = g / (1 + torch.exp(-g))
-        elif activation == "gelu_tanh":
-            a = 0.5 * g * (1 + torch.tanh(math.sqrt(2 / math.pi) * (g + 0.044715 * g * g * g)))
-        else:
+        if activation == "gelu":
             raise ValueError(activation)
+        a = self._act(g, activation)
+        if row_gate is not None:
+            a = a * torch.sigmoid(row_gate.float().reshape(-1, 1))
         out[:, :inner] = (a * u).to(out.dtype)
         if tail:
             out[:, inner:] = 0
@@ -166,7 +178,12 @@ class CpuKernels:
             vcache[blk, :, :, p % block_size] = v[r].reshape(kv_heads, value_dim)
 
     def sink_attention(self, q, out, heads, kv_heads, key_dim, value_dim, row_pos, row_seq, seq_slot, block_table,
-                       kcache, vcache, block_size, scale, window=0, keep_first=0, sink=True, gate=None, decode=False):
+                       kcache, vcache, block_size, scale, window=0, keep_first=0, sink=True, gate=None, decode=False,
+                       sink_values=None, maps=1):
+        if maps > 1:  # a cached key row holds the keys of `maps` key heads side by side; they share the value head
+            nb, g_heads, bs, wide = kcache.shape
+            kcache = kcache.reshape(nb, g_heads, bs, maps, key_dim).permute(0, 1, 3, 2, 4).reshape(nb, kv_heads, bs, key_dim)
+            vcache = vcache.repeat_interleave(maps, dim=1)
         for r in range(q.shape[0]):
             p = int(row_pos[r])
             slot = int(seq_slot[int(row_seq[r])])
@@ -177,9 +194,10 @@ class CpuKernels:
             for h in range(heads):
                 g = h // (heads // kv_heads)
                 s = (kk[:, g] @ q[r, h * key_dim : (h + 1) * key_dim].float()) * scale
-                m = torch.clamp(s.max(), min=0.0) if sink else s.max()
+                at = float(sink_values[h]) if sink_values is not None else 0.0
+                m = torch.clamp(s.max(), min=at) if sink else s.max()
                 e = torch.exp(s - m)
-                denom = e.sum() + (torch.exp(-m) if sink else 0.0)
+                denom = e.sum() + (torch.exp(at - m) if sink else 0.0)
                 o = (e[:, None] * vv[:, g]).sum(0) / denom
                 if gate is not None:
                     o = o * torch.sigmoid(gate[r, h].float())
@@ -308,8 +326,15 @@ class CpuKernels:
         for h in range(heads):
             out[:, h * out_head_stride : h * out_head_stride + size] = v[:, h].to(out.dtype)
 
+    def diff_combine(self, both, out, heads, kv_heads, value_dim, lam, eps, gain):
+        rows, group = both.shape[0], heads // kv_heads
+        a = both.float().reshape(rows, kv_heads, 2, group, value_dim)
+        o = (a[:, :, 0] - lam * a[:, :, 1]).reshape(rows, heads, value_dim)
+        o = o / torch.sqrt((o * o).mean(-1, keepdim=True) + eps) * gain
+        out.copy_(o.reshape(rows, heads * value_dim).to(out.dtype))
+
     def rotary_qkv(self, src, q_out, k_out, v_out, heads, kv_heads, key_dim, value_dim, dims, interleaved, freqs,
-                   magnitude, norm_eps, row_pos):
+                   magnitude, norm_eps, row_pos, value_width=0):
         rows = src.shape[0]
         n_rot = (heads + kv_heads) * key_dim
         turned = torch.empty((rows, n_rot), dtype=torch.float32)
@@ -358,23 +383,35 @@ class CpuKernels:
                 s.mul_(decay[:, None, :]).add_(vr[:, :, None] * kr[:, None, :])
                 out[r] = (s * qr[:, None, :]).sum(-1).reshape(-1)
 
-    def moe_route(self, logits, route, top, renormalize=False, correction=None, groups=0, keep=0):
-        s = torch.sigmoid(logits.float())
+    def moe_route(self, logits, route, top, renormalize=False, correction=None, groups=0, keep=0, scoring="sigmoid",
+                  group_mark="top2", renormalize_eps=0.0, identity=None):
+        s = torch.sigmoid(logits.float()) if scoring == "sigmoid" else torch.softmax(logits.float(), -1)
         c = s + correction if correction is not None else s
         experts = s.shape[1]
+        real = route.shape[1]
         route.fill_(-1.0)
+        if identity is not None:
+            identity.fill_(-1.0)
         for r in range(s.shape[0]):
             allowed = list(range(experts))
             if groups > 1 and keep < groups:
                 per = experts // groups
-                marks = [sum(sorted((float(c[r, e]) for e in range(g * per, (g + 1) * per)), reverse=True)[:2])
+                best = 1 if group_mark == "max" else 2
+                marks = [sum(sorted((float(c[r, e]) for e in range(g * per, (g + 1) * per)), reverse=True)[:best])
                          for g in range(groups)]
                 kept = sorted(range(groups), key=lambda g: (-marks[g], g))[:keep]
                 allowed = [e for e in allowed if e // per in kept]
             chosen = sorted(allowed, key=lambda e: (-float(c[r, e]), e))[:top]
-            total = sum(float(s[r, e]) for e in chosen) if renormalize else 1.0
+            total = sum(float(s[r, e]) for e in chosen) + renormalize_eps if renormalize else 1.0
             for e in chosen:
-                route[r, e] = s[r, e] / total
+                if e < real:
+                    route[r, e] = s[r, e] / total
+                else:
+                    identity[r, e - real] = s[r, e] / total
+
+    def moe_identity(self, h, weights, out):
+        w = torch.clamp(weights.float(), min=0.0).sum(-1, keepdim=True)
+        out += h.float() * w
 
     def moe_glu(self, gu, route, out, experts, ff, limit, weight_input=True, activation="clamped_swish"):
         rows = gu.shape[0]
