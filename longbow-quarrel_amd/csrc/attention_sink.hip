@@ -4,7 +4,8 @@
 // Row r of the step has position p = row_pos[r] in the sequence row_seq[r] and sees key t when t <= p and
 // (p - t < window or t < keep_first); window = 0: every t <= p.  Query head h reads kv head h / (nh / nkv).
 // score = q . k * scale; the softmax runs with a maximum that starts at 0 and a sum that starts at 1 when
-// there is a sink (a key of score 0 without a value), at -inf and 0 otherwise.  out = sum p_t v_t, times
+// there is a sink (a key of score 0 without a value; with `sinks`, a learned score a query head that is not scaled:
+// the maximum starts there), at -inf and 0 otherwise.  out = sum p_t v_t, times
 // sigmoid(gate[r, h]) where a gate is given.  Scores, probabilities and sums are 32-bit for either dtype of
 // q and the cache; the products run on the matrix cores in their 32-bit mode (v_mfma_f32_16x16x4_f32).
 //
@@ -13,6 +14,11 @@
 // what else is in the batch.
 //
 // Cache layout: K[block][kv head][offset][key size], V[block][kv head][value size][offset].
+//
+// `maps` > 1: nkv counts key heads of which every `maps` neighbours share one value head, and a cached key row
+// holds their keys side by side, K[block][value head][offset][map][key size], V[block][value head][...]: key head j
+// reads map j % maps of value head j / maps (differential attention: two score maps over the same values).
+// `out_f32`: out is 32-bit whatever the dtype of q and the cache.
 #include "common.h"
 
 namespace {
@@ -41,7 +47,15 @@ struct SinkArgs {
   // which a second launch merges in the order of the workgroups
   int ksplit;
   float* part;
+  int maps, out_f32;
+  const float* sinks;  // null: the sink's score is 0
 };
+
+template <typename T>
+__device__ inline void put_out(T* out, long long at, float v, int out_f32) {
+  if (out_f32) ((float*)out)[at] = v;
+  else out[at] = from_f32<T>(v);
+}
 
 constexpr int MAX_KD = 256;
 
@@ -74,6 +88,8 @@ __global__ __launch_bounds__(64 * SPLIT) void sink_tiles_kernel(const T* __restr
   // (tile row c: step row c / heads_per_tile, head c % heads_per_tile): their keys and values are read once.
   const int GH = a.heads_per_tile;
   const int hbase = blockIdx.y * GH, kvh = hbase / (a.nh / a.nkv);
+  const int nvh = a.nkv / a.maps, vh = kvh / a.maps, kmap = kvh % a.maps;  // value heads; this tile's, and its map
+  const long long krow = (long long)a.maps * a.KD;                          // a cached key row of one value head
   const int r0 = blockIdx.x * a.rows_per_tile;
   const int n_rows = min(a.rows_per_tile, a.rows - r0);
   const int HS = a.KD / 16, BS = a.BS;
@@ -92,7 +108,7 @@ __global__ __launch_bounds__(64 * SPLIT) void sink_tiles_kernel(const T* __restr
 
   // the sink is one more key of score 0 without a value: the first wavefront starts from it
   const bool with_sink = a.sink && wave == 0 && blockIdx.z == 0;
-  float m = with_sink ? 0.f : -INFINITY, l = with_sink ? 1.f : 0.f;
+  float m = with_sink ? (a.sinks != nullptr ? a.sinks[h] : 0.f) : -INFINITY, l = with_sink ? 1.f : 0.f;
   f32x4 o[HSV];  // o[dt][e]: row 4 g + e of the tile, value dimension 16 dt + c
 #pragma unroll
   for (int dt = 0; dt < HSV; ++dt) o[dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
@@ -122,7 +138,7 @@ __global__ __launch_bounds__(64 * SPLIT) void sink_tiles_kernel(const T* __restr
           st[kt] = (f32x4){0.f, 0.f, 0.f, 0.f};
           const int t = min(t0 + 16 * kt + c, pos_max);  // this lane's key as an operand row (clamped: finite, masked below)
           const long long blk = table[t / BS];
-          const T* kr = kcache + ((blk * a.nkv + kvh) * BS + t % BS) * (long long)a.KD + 4 * g;
+          const T* kr = kcache + ((blk * nvh + vh) * BS + t % BS) * krow + kmap * a.KD + 4 * g;
           if constexpr (HALF) {
             for (int sl = 0; sl < HS; ++sl) {
               const uint2 kv = *(const uint2*)(kr + sl * 16);
@@ -178,7 +194,7 @@ __global__ __launch_bounds__(64 * SPLIT) void sink_tiles_kernel(const T* __restr
           // V^T of this lane's dimension 16 dt + c at keys t0 + 16 kt + 4 g .. + 3 (within one block)
           const int t = min(t0 + 16 * kt + 4 * g, pos_max) & ~3;
           const long long blk = table[t / BS];
-          const T* vr = vcache + ((blk * a.nkv + kvh) * (long long)(HSV * 16) + c) * BS + t % BS;
+          const T* vr = vcache + ((blk * nvh + vh) * (long long)(HSV * 16) + c) * BS + t % BS;
           f32x4 vv[HSV];
 #pragma unroll
           for (int dt = 0; dt < HSV; ++dt) vv[dt] = ld4(vr + (long long)dt * 16 * BS);
@@ -239,9 +255,9 @@ __global__ __launch_bounds__(64 * SPLIT) void sink_tiles_kernel(const T* __restr
     if (row < n_rows) {
       float f = inv4[e];
       if (gate != nullptr) f /= 1.f + expf(-to_f32(gate[(long long)(r0 + row) * a.ldg + hh]));
-      T* orow = out + (long long)(r0 + row) * a.ldo + hh * (HSV * 16) + c;
+      const long long orow = (long long)(r0 + row) * a.ldo + hh * (HSV * 16) + c;
 #pragma unroll
-      for (int dt = 0; dt < HSV; ++dt) orow[dt * 16] = from_f32<T>(o[dt][e] * f);
+      for (int dt = 0; dt < HSV; ++dt) put_out(out, orow + dt * 16, o[dt][e] * f, a.out_f32);
     }
   }
 }
@@ -289,9 +305,9 @@ __global__ __launch_bounds__(64) void sink_merge_kernel(T* __restrict__ out, con
     if (row < n_rows) {
       float f = inv4[e];
       if (gate != nullptr) f /= 1.f + expf(-to_f32(gate[(long long)(r0 + row) * a.ldg + hh]));
-      T* orow = out + (long long)(r0 + row) * a.ldo + hh * (HSV * 16) + c;
+      const long long orow = (long long)(r0 + row) * a.ldo + hh * (HSV * 16) + c;
 #pragma unroll
-      for (int dt = 0; dt < HSV; ++dt) orow[dt * 16] = from_f32<T>(o[dt][e] * f);
+      for (int dt = 0; dt < HSV; ++dt) put_out(out, orow + dt * 16, o[dt][e] * f, a.out_f32);
     }
   }
 }
@@ -308,12 +324,13 @@ __global__ __launch_bounds__(64) void sink_rows_kernel(const T* __restrict__ q, 
   __shared__ float ps[64];
   __shared__ long long vbase[64];
   const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-  const int g = h / (a.nh / a.nkv), BS = a.BS, KD = a.KD, VD = a.VD;
+  const int kvh = h / (a.nh / a.nkv), BS = a.BS, KD = a.KD, VD = a.VD;
+  const int nvh = a.nkv / a.maps, g = kvh / a.maps, kmap = kvh % a.maps;  // g: the value head
   const int p = a.row_pos[r];
   const int lo = (a.window > 0 && p >= a.window) ? p - a.window + 1 : 0;
   const int* table = a.block_table + (long long)a.seq_slot[a.row_seq[r]] * a.bt_stride;
   for (int d = lane; d < KD; d += 64) qs[d] = to_f32(q[(long long)r * a.ldq + h * KD + d]);
-  float m = a.sink ? 0.f : -INFINITY, l = a.sink ? 1.f : 0.f;
+  float m = a.sink ? (a.sinks != nullptr ? a.sinks[h] : 0.f) : -INFINITY, l = a.sink ? 1.f : 0.f;
   float acc[MAX_DIM / 64];
 #pragma unroll
   for (int j = 0; j < MAX_DIM / 64; ++j) acc[j] = 0.f;
@@ -327,8 +344,8 @@ __global__ __launch_bounds__(64) void sink_rows_kernel(const T* __restrict__ q, 
     if (valid) {
       const long long blk = table[t / BS];
       const int off = t % BS;
-      vbase[lane] = (blk * a.nkv + g) * (long long)VD * BS + off;
-      const T* kr = kcache + ((blk * a.nkv + g) * BS + off) * (long long)KD;
+      vbase[lane] = (blk * nvh + g) * (long long)VD * BS + off;
+      const T* kr = kcache + ((blk * nvh + g) * BS + off) * (long long)a.maps * KD + kmap * KD;
       float dot = 0.f;
       for (int d = 0; d < KD; ++d) dot = fmaf(qs[d], to_f32(kr[d]), dot);
       s = dot * a.scale;
@@ -363,7 +380,7 @@ __global__ __launch_bounds__(64) void sink_rows_kernel(const T* __restrict__ q, 
 #pragma unroll
   for (int j = 0; j < MAX_DIM / 64; ++j) {
     const int d = lane + 64 * j;
-    if (d < VD) out[(long long)r * a.ldo + h * VD + d] = from_f32<T>(acc[j] * f);
+    if (d < VD) put_out(out, (long long)r * a.ldo + h * VD + d, acc[j] * f, a.out_f32);
   }
 }
 
@@ -489,7 +506,10 @@ extern "C" int lq_sink_attention(const void* q, int ldq, void* out, int ldo, con
                                  int batch, int nh, int nkv, int KD, int VD, const int* row_pos, const int* row_seq,
                                  const int* seq_slot, const int* block_table, int bt_stride, const void* kcache,
                                  const void* vcache, int block_size, float scale, int window, int keep_first, int sink,
-                                 int force_rows, int max_len, float* part, long long part_floats, hipStream_t stream) {
+                                 int force_rows, int max_len, float* part, long long part_floats, const float* sinks,
+                                 int maps, int out_f32, hipStream_t stream) {
+  LQ_REQUIRE(maps >= 1 && nkv % maps == 0, "sink_attention: %d key heads in runs of %d that share a value head", nkv, maps);
+  LQ_REQUIRE(sinks == nullptr || sink, "sink_attention: learned sink scores without a sink");
   LQ_REQUIRE(rows > 0 && batch > 0 && rows >= batch, "sink_attention: rows %d and sequences %d", rows, batch);
   LQ_REQUIRE(nh > 0 && nkv > 0 && nh % nkv == 0 && nh <= 65535, "sink_attention: %d heads over %d kv heads", nh, nkv);
   LQ_REQUIRE(KD > 0 && VD > 0 && KD <= MAX_DIM && VD <= MAX_DIM, "sink_attention: key size %d, value size %d", KD, VD);
@@ -502,6 +522,7 @@ extern "C" int lq_sink_attention(const void* q, int ldq, void* out, int ldo, con
   a.row_pos = row_pos, a.row_seq = row_seq, a.seq_slot = seq_slot, a.block_table = block_table;
   a.bt_stride = bt_stride, a.BS = block_size, a.scale = scale, a.window = window, a.keep_first = keep_first, a.sink = sink;
   a.ksplit = 1, a.part = nullptr;
+  a.maps = maps, a.out_f32 = out_f32 || dtype == LQ_F32, a.sinks = sinks;
   if (!force_rows) {
     const bool done = dtype == LQ_F32
                           ? launch_tiles<float>(q, out, gate, kcache, vcache, a, batch, max_len, part, part_floats, stream)
@@ -520,5 +541,50 @@ extern "C" int lq_sink_attention(const void* q, int ldq, void* out, int ldo, con
     sink_rows_kernel<bf16_t><<<grid, 64, 0, stream>>>((const bf16_t*)q, (bf16_t*)out, (const bf16_t*)gate,
                                                       (const bf16_t*)kcache, (const bf16_t*)vcache, a);
   LQ_CHECK_LAUNCH("sink_attention(rows)");
+  return 0;
+}
+
+
+namespace {
+
+// both [rows, kv heads, 2, group, VD] (32-bit: the two maps' results of the query heads of every key/value head),
+// out [rows, heads, VD]: o = a1 - lam a2, divided by its root mean square over VD (eps inside the root), times gain.
+// One wavefront a (row, head).
+template <typename T>
+__global__ __launch_bounds__(256) void diff_combine_kernel(const float* __restrict__ both, int ldb, T* __restrict__ out,
+                                                           int ldo, int nh, int group, int VD, float lam, float eps,
+                                                           float gain) {
+  const int r = blockIdx.x, lane = threadIdx.x & 63;
+  const int h = blockIdx.y * 4 + (threadIdx.x >> 6);
+  if (h >= nh) return;
+  const int kv = h / group, hg = h % group;
+  const float* a1 = both + (long long)r * ldb + ((long long)(kv * 2) * group + hg) * VD;
+  const float* a2 = a1 + (long long)group * VD;
+  float ss = 0.f;
+  for (int d = lane; d < VD; d += 64) {
+    const float o = a1[d] - lam * a2[d];
+    ss = fmaf(o, o, ss);
+  }
+  const float inv = gain / sqrtf(wave_sum(ss) / (float)VD + eps);
+  T* orow = out + (long long)r * ldo + (long long)h * VD;
+  for (int d = lane; d < VD; d += 64) orow[d] = from_f32<T>((a1[d] - lam * a2[d]) * inv);
+}
+
+}  // namespace
+
+extern "C" int lq_diff_combine(const float* both, int ldb, void* out, int out_dtype, int ldo, int rows, int nh, int nkv,
+                               int VD, float lam, float eps, float gain, hipStream_t stream) {
+  LQ_REQUIRE(rows > 0 && rows <= 0x7fffffff && nh > 0 && nkv > 0 && nh % nkv == 0 && VD > 0, "diff_combine: rows %d, %d heads over %d, size %d",
+             rows, nh, nkv, VD);
+  LQ_REQUIRE(ldb >= 2 * nh * VD && ldo >= nh * VD, "diff_combine: a row stride is smaller than its row");
+  LQ_REQUIRE(both && out, "diff_combine: null pointer");
+  LQ_REQUIRE(lq_ceil_div(nh, 4) <= 65535, "diff_combine: too many heads");
+  const dim3 grid(rows, lq_ceil_div(nh, 4));
+  if (out_dtype == LQ_F32)
+    diff_combine_kernel<float><<<grid, 256, 0, stream>>>(both, ldb, (float*)out, ldo, nh, nh / nkv, VD, lam, eps, gain);
+  else if (out_dtype == LQ_BF16)
+    diff_combine_kernel<bf16_t><<<grid, 256, 0, stream>>>(both, ldb, (bf16_t*)out, ldo, nh, nh / nkv, VD, lam, eps, gain);
+  else LQ_REQUIRE(false, "diff_combine: unknown dtype %d", out_dtype);
+  LQ_CHECK_LAUNCH("diff_combine");
   return 0;
 }

@@ -71,7 +71,7 @@ __global__ __launch_bounds__(128) void rotary_kernel(const float* __restrict__ s
 template <typename T>
 __global__ __launch_bounds__(256) void rotary_qkv_kernel(const float* __restrict__ src, int lds_, T* __restrict__ q_out,
                                                          int ldq, T* __restrict__ k_out, int ldk, T* __restrict__ v_out,
-                                                         int ldv, int H, int G, int D, int V, int dims, int interleaved,
+                                                         int ldv, int H, int G, int D, int VW, int dims, int interleaved,
                                                          const double* __restrict__ freqs, float mag, float norm_eps,
                                                          const int* __restrict__ row_pos) {
   extern __shared__ float cs[];  // cos[dims / 2], sin[dims / 2]
@@ -115,7 +115,7 @@ __global__ __launch_bounds__(256) void rotary_qkv_kernel(const float* __restrict
   }
   const float* vs = s + (H + G) * D;
   T* vo = v_out + (long long)r * ldv;
-  for (int e = blockIdx.y * blockDim.x + threadIdx.x; e < G * V; e += blockDim.x * gridDim.y) vo[e] = from_f32<T>(vs[e]);
+  for (int e = blockIdx.y * blockDim.x + threadIdx.x; e < VW; e += blockDim.x * gridDim.y) vo[e] = from_f32<T>(vs[e]);
 }
 
 // A product a head: out[r, h ohs + n] = sum_k x[r, h K + k] w[h, n, k], bfloat16 operands on
@@ -198,12 +198,15 @@ extern "C" int lq_rotary(const float* src, int lds_, void* out, int out_dtype, i
 extern "C" int lq_rotary_qkv(const float* src, int lds_, void* q_out, int ldq, void* k_out, int ldk, void* v_out, int ldv,
                              int out_dtype, int rows, int heads, int kv_heads, int key_dim, int value_dim, int dims,
                              int interleaved, const double* freqs, float magnitude, float norm_eps, const int* row_pos,
-                             hipStream_t stream) {
+                             int value_width, hipStream_t stream) {
+  // `value_width` > 0: so many value entries a row pass, in the place of kv_heads * value_dim (key heads that share
+  // a value head)
+  const int VW = value_width > 0 ? value_width : kv_heads * value_dim;
   LQ_REQUIRE(rows > 0 && heads > 0 && kv_heads > 0 && key_dim > 0 && value_dim > 0, "rotary_qkv: rows %d, heads %d and %d, sizes %d and %d",
              rows, heads, kv_heads, key_dim, value_dim);
   LQ_REQUIRE(dims >= 0 && dims % 2 == 0 && dims <= key_dim && dims <= 8192, "rotary_qkv: %d rotated entries of %d", dims, key_dim);
-  LQ_REQUIRE(lds_ >= (heads + kv_heads) * key_dim + kv_heads * value_dim && ldq >= heads * key_dim && ldk >= kv_heads * key_dim &&
-                 ldv >= kv_heads * value_dim, "rotary_qkv: a row stride is smaller than its row");
+  LQ_REQUIRE(lds_ >= (heads + kv_heads) * key_dim + VW && ldq >= heads * key_dim && ldk >= kv_heads * key_dim &&
+                 ldv >= VW, "rotary_qkv: a row stride is smaller than its row");
   LQ_REQUIRE(src && q_out && k_out && v_out && row_pos && (dims == 0 || freqs), "rotary_qkv: null pointer");
   const size_t lds_bytes = (size_t)dims * sizeof(float);
   // few rows (single tokens): a wavefront a head, so that no wavefront walks through its heads one after the other
@@ -211,11 +214,11 @@ extern "C" int lq_rotary_qkv(const float* src, int lds_, void* q_out, int ldq, v
   const dim3 grid(rows, share);
   if (out_dtype == LQ_F32)
     rotary_qkv_kernel<float><<<grid, 256, lds_bytes, stream>>>(src, lds_, (float*)q_out, ldq, (float*)k_out, ldk, (float*)v_out,
-                                                               ldv, heads, kv_heads, key_dim, value_dim, dims, interleaved,
+                                                               ldv, heads, kv_heads, key_dim, VW, dims, interleaved,
                                                                freqs, magnitude, norm_eps, row_pos);
   else if (out_dtype == LQ_BF16)
     rotary_qkv_kernel<bf16_t><<<grid, 256, lds_bytes, stream>>>(src, lds_, (bf16_t*)q_out, ldq, (bf16_t*)k_out, ldk,
-                                                                (bf16_t*)v_out, ldv, heads, kv_heads, key_dim, value_dim, dims,
+                                                                (bf16_t*)v_out, ldv, heads, kv_heads, key_dim, VW, dims,
                                                                 interleaved, freqs, magnitude, norm_eps, row_pos);
   else LQ_REQUIRE(false, "rotary_qkv: unknown dtype %d", out_dtype);
   LQ_CHECK_LAUNCH("rotary_qkv");

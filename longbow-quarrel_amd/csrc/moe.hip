@@ -9,16 +9,31 @@ namespace {
 // With `correction` the experts are chosen by s + correction[e]; the weights stay the scores s.  With `groups` > 1
 // the experts form that many equal groups of neighbours; a group's mark is the sum of its two largest choice scores
 // (of its one, in groups of one), and only experts of the `keep` groups with the largest marks (the lower index on a
-// tie) can be chosen.
+// tie) can be chosen.  `softmax`: s = softmax(z) over all E outputs in the sigmoid's place.  `mark_max`: a group's mark
+// is its largest choice score alone.  `renorm_eps` is added to the chosen scores' sum before the division.  The last
+// `n_ident` of the E outputs are experts without tensors: their weights go to `ident` [rows, n_ident] (-1: not
+// chosen) and `route` has the E - n_ident others.
 __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__ z, int ldz, float* __restrict__ route,
                                                        int rows, int E, int top, int renorm,
-                                                       const float* __restrict__ correction, int groups, int keep) {
+                                                       const float* __restrict__ correction, int groups, int keep,
+                                                       int softmax, int mark_max, float renorm_eps,
+                                                       float* __restrict__ ident, int n_ident) {
   const int r = blockIdx.x * 64 + threadIdx.x;
   if (r >= rows) return;
   const float* zr = z + (long long)r * ldz;
-  float* out = route + (long long)r * E;
-  for (int e = 0; e < E; ++e) out[e] = -1.f;
-  auto score = [&](int e) { return 1.f / (1.f + expf(-zr[e])); };
+  const int R = E - n_ident;  // experts with tensors
+  float* out_real = route + (long long)r * R;
+  float* out_ident = n_ident > 0 ? ident + (long long)r * n_ident : nullptr;
+  auto out = [&](int e) -> float& { return e < R ? out_real[e] : out_ident[e - R]; };
+  for (int e = 0; e < E; ++e) out(e) = -1.f;
+  float zmax = -INFINITY, inv_sum = 1.f;
+  if (softmax) {
+    for (int e = 0; e < E; ++e) zmax = fmaxf(zmax, zr[e]);
+    float sum = 0.f;
+    for (int e = 0; e < E; ++e) sum += expf(zr[e] - zmax);
+    inv_sum = 1.f / sum;
+  }
+  auto score = [&](int e) { return softmax ? expf(zr[e] - zmax) * inv_sum : 1.f / (1.f + expf(-zr[e])); };
   auto choice = [&](int e) { return correction != nullptr ? score(e) + correction[e] : score(e); };
   unsigned long long kept = ~0ull;  // bit g: group g may be chosen from
   const int per = groups > 1 ? E / groups : E;
@@ -35,7 +50,7 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__
           if (v > a) b = a, a = v;
           else if (v > b) b = v;
         }
-        const float mark = per > 1 ? a + b : a;
+        const float mark = per > 1 && !mark_max ? a + b : a;
         if (best < 0 || mark > bm) best = g, bm = mark;
       }
       if (best < 0) break;
@@ -47,19 +62,35 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__
     int best = -1;
     float bz = 0.f;
     for (int e = 0; e < E; ++e) {
-      if (out[e] >= 0.f) continue;  // chosen already
+      if (out(e) >= 0.f) continue;  // chosen already
       if (groups > 1 && !((kept >> (e / per)) & 1ull)) continue;
       const float v = choice(e);  // scores are compared, not logits: equal scores are a tie
       if (best < 0 || v > bz) best = e, bz = v;
     }
     if (best < 0) break;
     const float w = score(best);
-    out[best] = w == w ? w : 0.f;
-    total += out[best];
+    out(best) = w == w ? w : 0.f;
+    total += out(best);
   }
+  total += renorm_eps;
   if (renorm && total > 0.f)
     for (int e = 0; e < E; ++e)
-      if (out[e] >= 0.f) out[e] /= total;
+      if (out(e) >= 0.f) out(e) /= total;
+}
+
+// out[r, :] += h[r, :] * (the sum of the row's chosen identity experts' weights); weights [rows, n] (-1: not chosen)
+template <typename T>
+__global__ __launch_bounds__(256) void moe_identity_kernel(const T* __restrict__ h, int ldh,
+                                                           const float* __restrict__ weights, int n,
+                                                           float* __restrict__ out, int ldo, int width) {
+  const int r = blockIdx.x;
+  float w = 0.f;
+  for (int i = 0; i < n; ++i) {
+    const float v = weights[(long long)r * n + i];
+    if (v >= 0.f) w += v;
+  }
+  if (w == 0.f) return;
+  for (int c = threadIdx.x; c < width; c += 256) out[(long long)r * ldo + c] += w * to_f32(h[(long long)r * ldh + c]);
 }
 
 // gu [rows, E, 2, ff] (gate then up of every expert), route [rows, E]; out [rows, E, ff]:
@@ -165,16 +196,35 @@ __global__ __launch_bounds__(256) void moe_scatter_kernel(const float* __restric
 
 }  // namespace
 
+// `experts` counts every output of the router, the `n_ident` identity experts at its end included: route is
+// [rows, experts - n_ident], ident [rows, n_ident] (null without identity experts).
 extern "C" int lq_moe_route(const float* z, int ldz, float* route, int rows, int experts, int top, int renormalize,
-                            const float* correction, int groups, int keep, hipStream_t stream) {
+                            const float* correction, int groups, int keep, int softmax, int mark_max, float renorm_eps,
+                            float* ident, int n_ident, hipStream_t stream) {
   LQ_REQUIRE(groups >= 0 && (groups <= 1 || (groups <= 64 && experts % groups == 0 && keep >= 1 && keep <= groups)),
              "moe_route: %d experts in %d groups of which %d are kept", experts, groups, keep);
   LQ_REQUIRE(rows > 0 && experts > 0 && top >= 1 && top <= experts && ldz >= experts, "moe_route: rows %d, %d of %d experts",
              rows, top, experts);
+  LQ_REQUIRE(n_ident >= 0 && n_ident < experts && (n_ident == 0 || ident != nullptr) && renorm_eps >= 0.f,
+             "moe_route: %d identity experts of %d", n_ident, experts);
   LQ_REQUIRE(z && route, "moe_route: null pointer");
   moe_route_kernel<<<lq_ceil_div(rows, 64), 64, 0, stream>>>(z, ldz, route, rows, experts, top, renormalize, correction,
-                                                             groups, keep);
+                                                             groups, keep, softmax, mark_max, renorm_eps, ident, n_ident);
   LQ_CHECK_LAUNCH("moe_route");
+  return 0;
+}
+
+extern "C" int lq_moe_identity(const void* h, int dtype, int ldh, const float* weights, int n, float* out, int ldo, int rows,
+                               int width, hipStream_t stream) {
+  LQ_REQUIRE(rows > 0 && width > 0 && n > 0 && ldh >= width && ldo >= width, "moe_identity: rows %d, width %d, %d experts", rows,
+             width, n);
+  LQ_REQUIRE(h && weights && out, "moe_identity: null pointer");
+  if (dtype == LQ_F32)
+    moe_identity_kernel<float><<<rows, 256, 0, stream>>>((const float*)h, ldh, weights, n, out, ldo, width);
+  else if (dtype == LQ_BF16)
+    moe_identity_kernel<bf16_t><<<rows, 256, 0, stream>>>((const bf16_t*)h, ldh, weights, n, out, ldo, width);
+  else LQ_REQUIRE(false, "moe_identity: unknown dtype %d", dtype);
+  LQ_CHECK_LAUNCH("moe_identity");
   return 0;
 }
 

@@ -18,13 +18,16 @@ __device__ inline float gelu_tanh_f(float z) {
   return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
 }
 
-enum { ACT_NONE = 0, ACT_SILU = 1, ACT_RELU = 2, ACT_GELU_TANH = 3 };
+__device__ inline float gelu_erf_f(float z) { return 0.5f * z * (1.f + erff(z * 0.70710678118654752f)); }
+
+enum { ACT_NONE = 0, ACT_SILU = 1, ACT_RELU = 2, ACT_GELU_TANH = 3, ACT_GELU_ERF = 4 };
 
 __device__ inline float activate(float z, int act) {
   switch (act) {
     case ACT_SILU: return silu_f(z);
     case ACT_RELU: return fmaxf(z, 0.f);
     case ACT_GELU_TANH: return gelu_tanh_f(z);
+    case ACT_GELU_ERF: return gelu_erf_f(z);
     default: return z;
   }
 }
@@ -67,10 +70,13 @@ __global__ __launch_bounds__(256) void add_scaled_kernel(float* __restrict__ x, 
 }
 
 // out[r, c] = act(gu[r, c] + bias[c]) * (gu[r, I + c] + bias[I + c]); behind the I results `tail` more columns, a
-// one and then zeros: with the next product's bias as one more column of its weight, that product adds the bias itself
+// one and then zeros: with the next product's bias as one more column of its weight, that product adds the bias itself.
+// `row_gate` (a logit a row, stride ldrg): the row's results times its sigmoid.  `gated` 0: there is no up half,
+// out[r, c] = act(gu[r, c]).
 template <typename TI, typename TO>
 __global__ __launch_bounds__(256) void glu_kernel(const TI* __restrict__ gu, int ld, TO* __restrict__ out, int ldo,
-                                                  int I, int act, const float* __restrict__ bias, int tail) {
+                                                  int I, int act, const float* __restrict__ bias, int tail,
+                                                  const float* __restrict__ row_gate, int ldrg, int gated) {
   const int r = blockIdx.y;
   const int c = blockIdx.x * 256 + threadIdx.x;
   if (c >= I + tail) return;
@@ -78,8 +84,9 @@ __global__ __launch_bounds__(256) void glu_kernel(const TI* __restrict__ gu, int
     store_as<TO>(out + (long long)r * ldo + c, c == I ? 1.f : 0.f);
     return;
   }
-  float g = to_f32(gu[(long long)r * ld + c]), u = to_f32(gu[(long long)r * ld + I + c]);
+  float g = to_f32(gu[(long long)r * ld + c]), u = gated ? to_f32(gu[(long long)r * ld + I + c]) : 1.f;
   if (bias != nullptr) g += bias[c], u += bias[I + c];
+  if (row_gate != nullptr) u *= sigmoid_f(row_gate[(long long)r * ldrg]);
   store_as<TO>(out + (long long)r * ldo + c, activate(g, act) * u);
 }
 
@@ -990,9 +997,11 @@ extern "C" int lq_add_scaled(float* x, const float* delta, int pieces, long long
 }
 
 extern "C" int lq_glu(const void* gu, int in_dtype, int ld, void* out, int out_dtype, int ldo, int rows, int I, int act,
-                      const float* bias, int tail, hipStream_t stream) {
-  LQ_REQUIRE(rows > 0 && I > 0 && ld >= 2 * I && tail >= 0 && ldo >= I + tail, "glu: rows %d, inner %d, strides %d and %d", rows, I, ld, ldo);
-  LQ_REQUIRE(act >= ACT_SILU && act <= ACT_GELU_TANH, "glu: unknown activation %d", act);
+                      const float* bias, int tail, const float* row_gate, int ldrg, int gated, hipStream_t stream) {
+  LQ_REQUIRE(rows > 0 && I > 0 && ld >= (gated ? 2 : 1) * I && tail >= 0 && ldo >= I + tail, "glu: rows %d, inner %d, strides %d and %d", rows, I, ld, ldo);
+  LQ_REQUIRE(act >= ACT_SILU && act <= ACT_GELU_ERF, "glu: unknown activation %d", act);
+  LQ_REQUIRE(gated || (bias == nullptr && tail == 0), "glu: a plain activation takes no bias and leaves no tail");
+  LQ_REQUIRE(row_gate == nullptr || ldrg >= 1, "glu: the rows' gate needs a stride");
   LQ_REQUIRE(rows <= 65535 * 64, "glu: too many rows");
   LQ_REQUIRE(gu && out, "glu: null pointer");
   for (int r0 = 0; r0 < rows; r0 += 65535) {
@@ -1000,7 +1009,8 @@ extern "C" int lq_glu(const void* gu, int in_dtype, int ld, void* out, int out_d
     dim3 grid(lq_ceil_div(I + tail, 256), nr);
 #define LQ_GLU(TI, TO)                                                                                              \
   glu_kernel<TI, TO><<<grid, 256, 0, stream>>>((const TI*)gu + (long long)r0 * ld, ld, (TO*)out + (long long)r0 * ldo, \
-                                               ldo, I, act, bias, tail)
+                                               ldo, I, act, bias, tail,                                                 \
+                                               row_gate ? row_gate + (long long)r0 * ldrg : nullptr, ldrg, gated)
     if (in_dtype == LQ_F32 && out_dtype == LQ_F32) LQ_GLU(float, float);
     else if (in_dtype == LQ_F32 && out_dtype == LQ_BF16) LQ_GLU(float, bf16_t);
     else if (in_dtype == LQ_BF16 && out_dtype == LQ_BF16) LQ_GLU(bf16_t, bf16_t);

@@ -20,7 +20,7 @@ from .. import build as _build
 from .dry import query
 
 F32, BF16 = 0, 1
-ABI_VERSION = 9  # lq_abi_version() of the library these wrappers were written for
+ABI_VERSION = 10  # lq_abi_version() of the library these wrappers were written for
 _DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
 
 
@@ -723,21 +723,33 @@ class HipKernels:
                        block_table: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, block_size: int,
                        scale: float, window: int = 0, keep_first: int = 0, sink: bool = True,
                        gate: Optional[torch.Tensor] = None, decode: bool = False, max_len: int = 0,
-                       workspace: Optional[torch.Tensor] = None) -> None:
+                       workspace: Optional[torch.Tensor] = None, sink_values: Optional[torch.Tensor] = None,
+                       maps: int = 1) -> None:
         """Attention of the step's rows over their slots' cached keys: row at position p sees t <= p with
         p - t < window (0: all) or t < keep_first; with `sink` the softmax's denominator has one more term e^0;
         `gate` [rows, heads]: every head's result times the sigmoid of its entry.  Scores and probabilities
         are 32-bit.  out [rows, heads * value_dim] in the dtype of q and the cache.  `max_len` (an upper bound of the
         lengths) and `workspace` (`sink_attention_workspace(...)` floats) let a launch of single tokens share a tile's
-        keys out over several workgroups (bfloat16 runs only)."""
-        self._dev(q, out, gate, row_pos, row_seq, seq_slot, block_table, kcache, vcache)
+        keys out over several workgroups (bfloat16 runs only).  `sink_values` (float32 [heads]): the sink's term is
+        e^(its entry) for every query head, not e^0.  `maps` > 1: `kv_heads` counts key heads of which every `maps`
+        neighbours share a value head; the cache is K [blocks, kv_heads / maps, block_size, maps * key_dim] (a row
+        holds the neighbours' keys side by side) and V [blocks, kv_heads / maps, value_dim, block_size].  out may be
+        float32 in a bfloat16 run."""
+        self._dev(q, out, gate, row_pos, row_seq, seq_slot, block_table, kcache, vcache, sink_values)
         rows, batch = q.shape[0], seq_slot.numel()
         self._i32(row_pos, "row_pos", rows)
         self._i32(row_seq, "row_seq", rows)
-        self._check_paged(kcache, vcache, kv_heads, key_dim, value_dim, block_size, block_table, seq_slot, "sink_attention")
-        if q.shape[1] != heads * key_dim or tuple(out.shape) != (rows, heads * value_dim) or q.dtype != out.dtype \
-                or q.dtype != kcache.dtype:
+        if maps < 1 or kv_heads % maps:
+            raise KernelLibraryError(f"sink_attention: {kv_heads} key heads do not share value heads in runs of {maps}")
+        self._check_paged(kcache, vcache, kv_heads // maps, key_dim * maps, value_dim, block_size, block_table, seq_slot,
+                          "sink_attention")
+        if q.shape[1] != heads * key_dim or tuple(out.shape) != (rows, heads * value_dim) \
+                or out.dtype not in (q.dtype, torch.float32) or q.dtype != kcache.dtype:
             raise KernelLibraryError("sink_attention: q / out do not match the rows, the sizes or the cache's dtype")
+        if sink_values is not None:
+            if not sink:
+                raise KernelLibraryError("sink_attention: learned sink scores without a sink")
+            self._f32(sink_values, "sink_attention: sink_values", heads)
         if gate is not None and (tuple(gate.shape) != (rows, heads) or gate.dtype != q.dtype):
             raise KernelLibraryError("sink_attention: the gate is [rows, heads] in the dtype of q")
         if decode and rows != batch:
@@ -751,10 +763,25 @@ class HipKernels:
             _ptr(seq_slot), _ptr(block_table), c_int(int(block_table.stride(0))), _ptr(kcache), _ptr(vcache),
             c_int(block_size), c_float(scale), c_int(window), c_int(keep_first), c_int(1 if sink else 0),
             c_int(1 if self.force_generic else 0), c_int(max_len if workspace is not None else 0), _ptr(workspace),
-            c_longlong(0 if workspace is None else workspace.numel()), self.stream))
+            c_longlong(0 if workspace is None else workspace.numel()), _ptr(sink_values), c_int(maps),
+            c_int(1 if out.dtype == torch.float32 else 0), self.stream))
+
+    def diff_combine(self, both: torch.Tensor, out: torch.Tensor, heads: int, kv_heads: int, value_dim: int, lam: float,
+                     eps: float, gain: float) -> None:
+        """both float32 [rows, kv_heads, 2, heads / kv_heads, value_dim]: two attention results a query head over the
+        same values.  out [rows, heads * value_dim] = (a1 - lam a2) / sqrt(mean((a1 - lam a2)^2) + eps) * gain, the
+        mean over a head's value_dim."""
+        rows, nb, ldb = self._mat(both, "diff_combine: both")
+        ro, no, ldo = self._mat(out, "diff_combine: out")
+        self._f32(both, "diff_combine: both")
+        if heads % kv_heads or nb != 2 * heads * value_dim or (ro, no) != (rows, heads * value_dim):
+            raise KernelLibraryError("diff_combine: both [rows, 2 heads value_dim] and out [rows, heads value_dim]")
+        self._check(self.lib.lq_diff_combine(_ptr(both), c_int(ldb), _ptr(out), c_int(_code(out)), c_int(ldo), c_int(rows),
+                                             c_int(heads), c_int(kv_heads), c_int(value_dim), c_float(lam), c_float(eps),
+                                             c_float(gain), self.stream))
 
     # ------------------------------------------------------------------ recurrent mixers and what surrounds them
-    _ACTIVATIONS = {"none": 0, "silu": 1, "relu": 2, "gelu_tanh": 3}
+    _ACTIVATIONS = {"none": 0, "silu": 1, "relu": 2, "gelu_tanh": 3, "gelu": 4}
 
     @staticmethod
     def _f32(t: torch.Tensor, what: str, n: Optional[int] = None) -> None:
@@ -788,21 +815,39 @@ class HipKernels:
         self._check(self.lib.lq_add_scaled(_ptr(x), _ptr(delta), c_int(pieces), c_longlong(stride), c_float(scale),
                                            c_longlong(x.numel()), self.stream))
 
+    def activation(self, x: torch.Tensor, out: torch.Tensor, activation: str) -> None:
+        """out = act(x), element by element in 32-bit; act: silu, relu, gelu_tanh or gelu (the exact one, with the error
+        function)."""
+        rows, inner, ld = self._mat(x, "activation: x")
+        ro, wide, ldo = self._mat(out, "activation: out")
+        if (ro, wide) != (rows, inner) or activation not in self._ACTIVATIONS or activation == "none":
+            raise KernelLibraryError(f"activation: x {tuple(x.shape)}, out {tuple(out.shape)}, activation {activation!r}")
+        self._check(self.lib.lq_glu(_ptr(x), c_int(_code(x)), c_int(ld), _ptr(out), c_int(_code(out)), c_int(ldo),
+                                    c_int(rows), c_int(inner), c_int(self._ACTIVATIONS[activation]), _ptr(None), c_int(0),
+                                    _ptr(None), c_int(0), c_int(0), self.stream))
+
     def glu(self, gate_up: torch.Tensor, out: torch.Tensor, activation: str, bias: Optional[torch.Tensor] = None,
-            tail: int = 0) -> None:
+            tail: int = 0, row_gate: Optional[torch.Tensor] = None) -> None:
         """out = act(gate) * up for gate_up [rows, 2 * inner] = [gate | up]; act: silu, relu or gelu_tanh.  `bias`
         (float32 [2 * inner]) is added to gate and up first.  With `tail` out is [rows, inner + tail] and its last
-        columns become a one and then zeros (the next product's bias rides as one more column of its weight)."""
+        columns become a one and then zeros (the next product's bias rides as one more column of its weight).
+        `row_gate` (float32 [rows, 1], any row stride): a row's results times the sigmoid of its entry."""
         rows, two, ld = self._mat(gate_up, "glu: gate_up")
         ro, wide, ldo = self._mat(out, "glu: out")
         inner = wide - tail
-        if ro != rows or tail < 0 or two != 2 * inner or activation not in self._ACTIVATIONS or activation == "none":
+        if ro != rows or tail < 0 or two != 2 * inner or activation not in self._ACTIVATIONS \
+                or activation in ("none", "gelu"):
             raise KernelLibraryError(f"glu: gate_up {tuple(gate_up.shape)}, out {tuple(out.shape)}, activation {activation!r}")
         if bias is not None:
             self._f32(bias, "glu: bias", 2 * inner)
+        ldrg = 0
+        if row_gate is not None:
+            rg, one, ldrg = self._mat(row_gate, "glu: row_gate")
+            if (rg, one) != (rows, 1) or row_gate.dtype != torch.float32:
+                raise KernelLibraryError("glu: the rows' gate is float32 [rows, 1]")
         self._check(self.lib.lq_glu(_ptr(gate_up), c_int(_code(gate_up)), c_int(ld), _ptr(out), c_int(_code(out)),
                                     c_int(ldo), c_int(rows), c_int(inner), c_int(self._ACTIVATIONS[activation]),
-                                    _ptr(bias), c_int(tail), self.stream))
+                                    _ptr(bias), c_int(tail), _ptr(row_gate), c_int(ldrg), c_int(1), self.stream))
 
     def causal_conv(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], state: torch.Tensor,
                     out: torch.Tensor, row_pos: torch.Tensor, row_seq: torch.Tensor, seq_slot: torch.Tensor,
@@ -1010,19 +1055,21 @@ class HipKernels:
     def rotary_qkv(self, src: torch.Tensor, q_out: torch.Tensor, k_out: torch.Tensor, v_out: torch.Tensor, heads: int,
                    kv_heads: int, key_dim: int, value_dim: int, dims: int, interleaved: bool,
                    freqs: Optional[torch.Tensor], magnitude: float, norm_eps: Optional[float],
-                   row_pos: torch.Tensor) -> None:
+                   row_pos: torch.Tensor, value_width: int = 0) -> None:
         """src float32 [rows, (heads + kv_heads) key_dim + kv_heads value_dim] = [queries | keys | values] goes to
         q_out, k_out and v_out in their dtype: of every query and key head the first `dims` entries rotated by
         row_pos[r] * freqs (float64 [dims / 2]; pairing and magnitude as `rotary`), then, with `norm_eps` not None,
-        the head divided by its root mean square over key_dim (eps inside the root); values pass."""
+        the head divided by its root mean square over key_dim (eps inside the root); values pass.  `value_width` > 0:
+        the values are so many entries a row, not kv_heads * value_dim (key heads that share a value head)."""
         rows, ns, lds = self._mat(src, "rotary_qkv: src")
         rq, nq, ldq = self._mat(q_out, "rotary_qkv: q")
         rk, nk, ldk = self._mat(k_out, "rotary_qkv: k")
         rv, nv, ldv = self._mat(v_out, "rotary_qkv: v")
         self._i32(row_pos, "row_pos", rows)
-        if src.dtype != torch.float32 or ns != (heads + kv_heads) * key_dim + kv_heads * value_dim \
+        vw = value_width if value_width > 0 else kv_heads * value_dim
+        if src.dtype != torch.float32 or ns != (heads + kv_heads) * key_dim + vw \
                 or (rq, nq) != (rows, heads * key_dim) or (rk, nk) != (rows, kv_heads * key_dim) \
-                or (rv, nv) != (rows, kv_heads * value_dim) or not q_out.dtype == k_out.dtype == v_out.dtype:
+                or (rv, nv) != (rows, vw) or not q_out.dtype == k_out.dtype == v_out.dtype:
             raise KernelLibraryError("rotary_qkv: src float32 [rows, q | k | v], outputs of one dtype with their sizes")
         if dims and (freqs is None or freqs.dtype != torch.float64 or not freqs.is_cuda or not freqs.is_contiguous()
                      or freqs.numel() != dims // 2):
@@ -1032,7 +1079,7 @@ class HipKernels:
                                            c_int(kv_heads), c_int(key_dim), c_int(value_dim), c_int(dims),
                                            c_int(1 if interleaved else 0), _ptr(freqs if dims else None),
                                            c_float(magnitude), c_float(-1.0 if norm_eps is None else norm_eps),
-                                           _ptr(row_pos), self.stream))
+                                           _ptr(row_pos), c_int(value_width), self.stream))
 
     def postnorm_residual(self, x: torch.Tensor, y: torch.Tensor, scales, weight: torch.Tensor, eps: float,
                           extra: Optional[torch.Tensor] = None, next_weight: Optional[torch.Tensor] = None,
@@ -1133,20 +1180,44 @@ class HipKernels:
                                          c_longlong(0 if workspace is None else workspace.numel()), self.stream))
 
     def moe_route(self, logits: torch.Tensor, route: torch.Tensor, top: int, renormalize: bool = False,
-                  correction: Optional[torch.Tensor] = None, groups: int = 0, keep: int = 0) -> None:
+                  correction: Optional[torch.Tensor] = None, groups: int = 0, keep: int = 0, scoring: str = "sigmoid",
+                  group_mark: str = "top2", renormalize_eps: float = 0.0,
+                  identity: Optional[torch.Tensor] = None) -> None:
         """route[r, e] = sigmoid(logits[r, e]) for the `top` experts with the largest scores (the lower index on a
         tie; divided by the chosen scores' sum with `renormalize`), -1 for the others.  float32.  With `correction`
         (float32 [experts]) the choice goes by score + correction, the weights stay the scores.  With `groups` > 1
         the experts form that many equal groups of neighbours and only experts of the `keep` groups whose two largest
-        choice scores sum highest can be chosen."""
+        choice scores sum highest can be chosen (`group_mark` "max": whose largest choice score is highest).
+        `scoring` "softmax": the scores are softmax(logits) over all columns.  `renormalize_eps` is added to the chosen
+        scores' sum before the division.  `identity` (float32 [rows, n]): the last n columns of the logits are experts
+        without tensors; their weights (-1: not chosen) go there and `route` is [rows, experts - n]."""
         rows, experts, ldz = self._mat(logits, "moe_route: logits")
         self._f32(logits, "moe_route: logits")
-        self._f32(route, "moe_route: route", rows * experts)
+        n_ident = 0
+        if identity is not None:
+            n_ident = identity.shape[-1]
+            self._f32(identity, "moe_route: identity", rows * n_ident)
+        if scoring not in ("sigmoid", "softmax") or group_mark not in ("top2", "max"):
+            raise KernelLibraryError(f"moe_route: scoring {scoring!r}, group_mark {group_mark!r}")
+        self._f32(route, "moe_route: route", rows * (experts - n_ident))
         if correction is not None:
             self._f32(correction, "moe_route: correction", experts)
         self._check(self.lib.lq_moe_route(_ptr(logits), c_int(ldz), _ptr(route), c_int(rows), c_int(experts), c_int(top),
                                           c_int(1 if renormalize else 0), _ptr(correction), c_int(groups), c_int(keep),
-                                          self.stream))
+                                          c_int(1 if scoring == "softmax" else 0), c_int(1 if group_mark == "max" else 0),
+                                          c_float(renormalize_eps), _ptr(identity), c_int(n_ident), self.stream))
+
+    def moe_identity(self, h: torch.Tensor, weights: torch.Tensor, out: torch.Tensor) -> None:
+        """out [rows, width] (float32) += h * (the sum of the row's entries of `weights` [rows, n] that are not
+        negative): the share of experts that hand their input on."""
+        rows, width, ldh = self._mat(h, "moe_identity: h")
+        ro, wo, ldo = self._mat(out, "moe_identity: out")
+        self._f32(out, "moe_identity: out")
+        if (ro, wo) != (rows, width) or weights.dim() != 2 or weights.shape[0] != rows:
+            raise KernelLibraryError("moe_identity: h and out [rows, width], weights [rows, n]")
+        self._f32(weights, "moe_identity: weights", rows * weights.shape[1])
+        self._check(self.lib.lq_moe_identity(_ptr(h), c_int(_code(h)), c_int(ldh), _ptr(weights), c_int(weights.shape[1]),
+                                             _ptr(out), c_int(ldo), c_int(rows), c_int(width), self.stream))
 
     def moe_glu(self, gu: torch.Tensor, route: torch.Tensor, out: torch.Tensor, experts: int, ff: int, limit: float,
                 weight_input: bool = True, activation: str = "clamped_swish") -> None:
