@@ -86,11 +86,15 @@ def rotate_half(x: torch.Tensor, rot: Optional[dict]) -> torch.Tensor:
     return out
 
 
-def window_mask(T: int, size: int) -> torch.Tensor:
-    """[T, T] true where row i sees column j: 0 <= i - j < size."""
+def window_mask(T: int, size: Optional[int]) -> torch.Tensor:
+    """[T, T] true where row i sees column j: 0 <= i - j < size (no size: every j <= i)."""
     i = torch.arange(T)[:, None]
     j = torch.arange(T)[None, :]
-    return (j <= i) & (i - j < size)
+    return (j <= i) & (i - j < (T if size is None else size))
+
+
+def window_of(m: dict) -> Optional[int]:
+    return m["mask"]["size"] if m.get("mask") else None
 
 
 def softmax_rows(score: torch.Tensor, seen: torch.Tensor, sink: Optional[float] = None) -> torch.Tensor:
@@ -112,7 +116,7 @@ def sink_attention(h, m: dict, w: Dict[str, torch.Tensor], p: str, eps: float, r
     k = rotate_half((h @ w[p + ".k"].T).view(T, G, d), m.get("rot"))
     q, k = rnd(rms(q, eps), rounding), rnd(rms(k, eps), rounding)
     v = rnd((h @ w[p + ".v"].T).view(T, G, vd), rounding)
-    seen = window_mask(T, m["mask"]["size"])
+    seen = window_mask(T, window_of(m))
     out = torch.zeros(T, H, vd, dtype=F)
     for n in range(H):
         g = n // (H // G)
@@ -133,7 +137,7 @@ def differential_attention(h, m: dict, w: Dict[str, torch.Tensor], p: str, eps: 
     q = rnd(rotate_half((h @ w[p + ".q"].T).view(T, H, 2, d), m.get("rot")), rounding)
     k = rnd(rotate_half((h @ w[p + ".k"].T).view(T, G, 2, d), m.get("rot")), rounding)
     v = rnd((h @ w[p + ".v"].T).view(T, G, vd), rounding)
-    seen = window_mask(T, m["mask"]["size"])
+    seen = window_mask(T, window_of(m))
     lam = differential_lambda(w, p, m["diff"])
     out = torch.zeros(T, H, vd, dtype=F)
     for n in range(H):
