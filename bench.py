@@ -35,6 +35,9 @@ such that a token's two experts together are as wide as the Llama shape's feed-f
 `--design mifidra`: the same for the design of softmax attention and the gated delta rule side by side (a decay for
 every key channel), with gated units and mixtures of experts in turn; beside the Llama shape and beside the Vafodra
 design of the same sizes, whose gated delta rule (one decay a head) and attention are the closest kernels.
+`--design sofinex`: the same for the design of differential attention under a sliding window, in turn with layers of
+windowed attention with a learned sink beside the gated delta rule; beside the Llama shape and beside the Mifidra
+design of the same sizes (the closest: the same attention kernel and delta rule, experts chosen within groups).
 """
 from __future__ import annotations
 
@@ -153,6 +156,32 @@ def mifidra_config(width: int, layers: int, vocab: int) -> dict:
             "width": width}
 
 
+def sofinex_config(width: int, layers: int, vocab: int) -> dict:
+    """Layer sizes of a real model for the design.  Even layers: attention heads of 128 under a window of 1 024 (a
+    fourth as many key/value heads, 64 entries rotated under YaRN, a learned sink) beside delta-rule heads of
+    128 x 128 (half as many q/k heads, four taps, bottlenecks of 64), and two matrices around the exact gelu, 5.25
+    times the width (the weights of a gated unit of 3.5).  Odd layers: differential attention, half as many heads
+    with two maps of 128 each and values of 256 under a window of 2 048, 64 entries rotated with frequencies blended
+    by wavelength; 6 experts and 2 identity experts in 4 groups of which 2 are kept, 2 a token, each 1.25 times the
+    width, beside a gated shared expert as wide as the model.  No stretch of layers runs twice."""
+    heads = width // 128
+    yarn = {"base": 10000.0, "dims": 64, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}
+    blend = {"base": 500000.0, "dims": 64, "scaling": {"factor": 8.0, "original": 8192, "low": 1.0, "high": 4.0}}
+    left = {"dim": 128, "vdim": 128, "heads": heads, "kv_heads": max(1, heads // 4), "scale": 128 ** -0.5,
+            "mask": {"size": 1024}, "rot": yarn}
+    right = {"conv": 4, "dim": 128, "vdim": 128, "heads": heads, "kv_heads": max(1, heads // 2), "decay_rank": 64,
+             "gate_rank": 64}
+    diff = {"dim": 128, "vdim": 256, "heads": max(1, heads // 2), "kv_heads": max(1, heads // 8), "scale": 128 ** -0.5,
+            "mask": {"size": 2048}, "rot": blend, "diff": 0.5}
+    dense = {"kind": "dense", "ff": width * 21 // 4}
+    moe = {"kind": "moe", "expert": {"ff": width * 5 // 4}, "shared": {"ff": width},
+           "router": {"experts": 6, "identity": 2, "top": 2, "groups": {"count": 4, "keep": 2}}}
+    made = [{"type": "attention", "mixer": diff, "mlp": moe} if i % 2 else
+            {"type": "parallel", "mixer": {"left": left, "right": right}, "mlp": dense} for i in range(layers)]
+    return {"architecture": "Sofinex", "embedding": {"scale": 1.0}, "layers": made, "norm": {"eps": 1e-5},
+            "vocab": vocab, "width": width}
+
+
 def design_run(args) -> int:
     import torch
 
@@ -169,8 +198,10 @@ def design_run(args) -> int:
                      num_attention_heads=width // 128, num_key_value_heads=max(1, width // 512), vocab_size=vocab)
         made = {"vafodra": lambda: lq.VafodraConfig.from_dict(vafodra_config(width, layers, vocab)),
                 "vupelorn": lambda: lq.VupelornConfig.from_dict(vupelorn_config(width, layers, vocab)),
-                "mifidra": lambda: lq.MifidraConfig.from_dict(mifidra_config(width, layers, vocab))}
-        beside = [("vafodra", made["vafodra"]())] if args.design == "mifidra" else []
+                "mifidra": lambda: lq.MifidraConfig.from_dict(mifidra_config(width, layers, vocab)),
+                "sofinex": lambda: lq.SofinexConfig.from_dict(sofinex_config(width, layers, vocab))}
+        closest = {"mifidra": "vafodra", "sofinex": "mifidra"}.get(args.design)
+        beside = [(closest, made[closest]())] if closest else []
         for name, config in [(args.design, made[args.design]())] + beside + [("llama", lq.LlamaConfig.from_dict(llama))]:
             engine = lq.random_engine(config, seed=0, dtype=args.dtype, max_tokens=batch * 4096 + n_prefill + 64,
                                       max_slots=batch + 1, max_sequence_tokens=max(4096, n_prefill))
@@ -230,7 +261,7 @@ def design_run(args) -> int:
             del engine, backend, timed
             torch.cuda.empty_cache()
     print(json.dumps({"metric": f"prefill and decode tok/s of the {args.design.capitalize()} design beside the Llama shape "
-                                "of equal size" + (" and the Vafodra design" if args.design == "mifidra" else ""),
+                                "of equal size" + (f" and the {closest.capitalize()} design" if closest else ""),
                       "dtype": args.dtype, "data": "synthetic: random weights from a seed, uniform random token ids",
                       "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "results": results}), flush=True)
     return 0
@@ -260,7 +291,7 @@ def main() -> int:
                     help="float32: the true 32-bit path (use --layers with the larger shapes)")
     ap.add_argument("--context", type=int, default=0,
                     help="tokens a sequence may hold (default: the shape's 8192); for decoding over longer prompts")
-    ap.add_argument("--design", choices=["vafodra", "vupelorn", "mifidra"], default=None,
+    ap.add_argument("--design", choices=["vafodra", "vupelorn", "mifidra", "sofinex"], default=None,
                     help="measure this design beside the Llama shape of equal size instead of the default workload")
     ap.add_argument("--design-widths", default="2048,4096", help="model widths of --design, with commas between them")
     args = ap.parse_args()
