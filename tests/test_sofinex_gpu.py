@@ -179,12 +179,18 @@ def test_rotation_of_half_split_pairs_of_every_map(kn, dtype, sizes):
 
 
 def test_exact_gelu_and_a_gate_a_row_on_a_gated_unit(kn):
-    rows, inner = 33, 70
-    x = rnd(rows, inner, seed=1, std=2.5)
-    for dtype in (torch.float32, torch.bfloat16):
-        out = torch.zeros((rows, inner), dtype=dtype, device=DEV)
-        kn.activation(dev(x), out, "gelu")
-        assert sc.err(out, ps.gelu_erf(x.double())) < (2e-6 if dtype == torch.float32 else 1e-2)
+    rows = 33
+    for inner in (70, 72, 1024):  # (columns in fours go four a thread)
+        x = rnd(rows, inner, seed=1, std=2.5)
+        for dtype in (torch.float32, torch.bfloat16):
+            out = torch.zeros((rows, inner), dtype=dtype, device=DEV)
+            kn.activation(dev(x), out, "gelu")
+            assert sc.err(out, ps.gelu_erf(x.double())) < (2e-6 if dtype == torch.float32 else 1e-2)
+            wide = torch.full((rows, inner + 8), 7.0, dtype=dtype, device=DEV)  # rows with a stride of their own
+            kn.activation(dev(torch.cat([x, x[:, :4]], 1))[:, :inner], wide[:, :inner], "silu")
+            assert sc.err(wide[:, :inner], ps.silu(x.double())) < (2e-6 if dtype == torch.float32 else 1e-2)
+            assert bool((wide[:, inner:] == 7.0).all())
+    inner = 70
     # the tanh form is another function, further off than the kernel's limit above
     xd = x.double()
     tanh_form = 0.5 * xd * (1 + torch.tanh(math.sqrt(2 / math.pi) * (xd + 0.044715 * xd ** 3)))
