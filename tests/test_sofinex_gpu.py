@@ -129,6 +129,43 @@ def test_windowed_attention_with_a_learned_sink_and_maps_that_share_values(kn, s
         kn.force_generic = False
 
 
+@pytest.mark.parametrize("sizes", [
+    # query heads, key heads, maps, key size, value size, window, learned sink
+    (4, 2, 1, 32, 48, 0, True), (4, 2, 1, 32, 48, 700, True), (8, 4, 2, 16, 80, 0, False), (6, 2, 2, 48, 96, 520, False),
+])
+def test_single_tokens_whose_keys_are_shared_out_over_workgroups(kn, sizes):
+    """A bfloat16 step of single tokens over many cached keys: a tile's keys go to several workgroups and a second
+    launch merges them.  The sink's term must count once (the first workgroup's first wavefront starts from it), and
+    every workgroup must read its map's half of the cached key rows."""
+    H, G, maps, D, P, window, sink = sizes
+    T, dtype = 1500, torch.bfloat16
+    Gv = G // maps
+    q, k, v = rnd(T, H, D, seed=1), rnd(T, G, D, seed=2), rnd(T, Gv, P, seed=3)
+    sinks = rnd(H, seed=4, std=1.0) + 3.0 if sink else None  # (a sink that takes a large share of the weight)
+    q, k, v = (t.to(dtype).double() for t in (q, k, v))
+    scale = 1.0 / math.sqrt(D)
+    want = plain_maps(q, k, v, scale, window if window else T, None if sinks is None else sinks.double()).reshape(T, H * P)
+    if sink:
+        assert sc.err(plain_maps(q, k, v, scale, window if window else T).reshape(T, H * P), want) > 5e-2
+    cache = Paged(T, Gv, maps * D, P, dtype, seed=5)
+    pos, seq, slot = i32(range(T)), i32([0] * T), i32([0])
+    kn.kv_store(dev(k.reshape(T, -1), dtype), dev(v.reshape(T, -1), dtype), Gv, maps * D, P, pos, seq, slot, cache.table,
+                cache.k, cache.v, 64)
+    qd = dev(q.reshape(T, -1), dtype)
+    more = dict(window=window, keep_first=0, sink=sink, maps=maps)
+    if sink:
+        more["sink_values"] = dev(sinks)
+    need = kn.sink_attention_workspace(dtype, 1, 1, H, G, D, P, 64, window, 0, T)
+    assert need > 0
+    scratch = torch.zeros(need, device=DEV)
+    for r in (T - 1, 1100, 800, 767, 700):
+        for out_dtype in (torch.float32, dtype):
+            one = torch.zeros((1, H * P), dtype=out_dtype, device=DEV)
+            kn.sink_attention(qd[r : r + 1], one, H, G, D, P, i32([r]), i32([0]), slot, cache.table, cache.k, cache.v, 64,
+                              scale, decode=True, max_len=T, workspace=scratch, **more)
+            assert sc.err(one[0], want[r]) < (2e-5 if out_dtype == torch.float32 else 1e-2), (r, out_dtype)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("sizes", [(4, 2, 48), (3, 3, 7), (6, 1, 96), (2, 1, 130), (8, 4, 16)])
 def test_difference_of_two_maps_and_its_norm(kn, sizes, dtype):
