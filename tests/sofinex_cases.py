@@ -76,7 +76,7 @@ def _config(vocab, width, eps, emb_scale, layers, loop=None):
 # run three times
 CFG_A = _config(173, 80, 1e-6, 3.0, [
     _parallel(_heads(6, 2, 24, 16, 0.3, 20, 3000.0, 16, YARN), _delta(4, 2, 12, 20, 4, 6, 10), _dense(56)),
-    _diff_layer(_heads(2, 2, 16, 40, 0.25, 70, 500.0, 8, LLAMA, diff=0.6), _moe(4, 2, 2, 24, (3, 1), 40)),
+    _diff_layer(_heads(2, 2, 16, 40, 0.25, 70, 500.0, 8, LLAMA, diff=0.65), _moe(4, 2, 2, 24, (3, 1), 40)),
     _parallel(_heads(4, 1, 32, 32, 0.15, 130, 10000.0, 8), _delta(3, 1, 16, 16, 3, 8, 8), None),
     _diff_layer(_heads(3, 1, 8, 24, 0.35, 1000, 100.0, None, {"factor": 2.0, "original": 16, "low": 2.0, "high": 8.0},
                        diff=0.3), _moe(5, 1, 3, 16, (2, 2))),
@@ -114,7 +114,7 @@ CFG_MOE = _config(60, 48, 1e-6, 2.0, [
     _diff_layer(_heads(1, 1, 8, 8, 0.3, 10, 100.0, diff=0.5), _moe(9, 3, 3, 20, (4, 2), 28))])
 CFG_LOOP = _config(60, 48, 1e-6, 1.5, [
     _parallel(_heads(2, 1, 8, 8, 0.3, 30, 100.0), _delta(1, 1, 8, 8, 2, 2, 2), _dense(24)),
-    _diff_layer(_heads(1, 1, 16, 8, 0.2, 25, 100.0, diff=0.6), None),
+    _diff_layer(_heads(1, 1, 16, 8, 0.2, 25, 100.0, diff=0.65), None),
     _parallel(_heads(2, 2, 8, 16, 0.3, 66, 100.0), _delta(2, 1, 8, 8, 2, 3, 3), _dense(16)),
 ], loop=(0, 2, 3))
 CONFIGS = {"a": CFG_A, "b": CFG_B, "c": CFG_C, "diff": CFG_DIFF, "sink": CFG_SINK, "delta": CFG_DELTA,
